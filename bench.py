@@ -1,0 +1,200 @@
+#!/usr/bin/env python3
+"""Benchmark of the routed-expert FFN (B1, E-W4A8-v1) on one MI355X.
+
+One step = one pass of the hot path (plan -> FC1 + SwiGLU + requant -> FC2 -> combine) over one
+batch of synthetic, device-resident input. Prints ONE JSON line: routed tokens/s per MoE layer for
+the 128-token decode/verify layer (256 experts, H 4096, I 2048, top-8), its HBM roofline, the CPU
+restatement of the reference timed on the host's cores, and, unless --no-prefill, the same
+measurement for the 8192-token prefill chunk against the MFMA peak.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "oracle"))
+
+HBM_PEAK_GBS = 8000.0           # MI355X HBM3E, published
+MFMA_FP8_PEAK_TFLOPS = 5000.0   # dense FP8 (an FP8 x FP4 block-scaled MFMA issues at the FP8 rate)
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def stage(wl, torch, dev):
+    """Workload arrays as device tensors."""
+    return dict(payload=torch.from_numpy(wl.payload).to(dev), scales=torch.from_numpy(wl.scales).to(dev),
+                ids=torch.from_numpy(wl.ids).to(dev), weights=torch.from_numpy(wl.weights).to(dev),
+                out=torch.empty((wl.rows, 4096), dtype=torch.int16, device=dev))
+
+
+def build_layer(wl, torch, dev, b1):
+    """Generate the canonical rank pools, upload them, prepare the layer, drop the canonical copies."""
+    t0 = time.time()
+    pools = wl.pools()
+    log(f"[bench] generated {len(pools)} rank pools in {time.time() - t0:.1f}s")
+    devs = [torch.from_numpy(p).to(dev) for p in pools]
+    torch.cuda.synchronize()
+    if len(devs) == 1:
+        layer = b1.Layer(devs[0].data_ptr(), devs[0].numel(), 0)
+    else:
+        layer = b1.Layer.full([d.data_ptr() for d in devs], devs[0].numel())
+    del devs
+    torch.cuda.empty_cache()
+    return layer, pools
+
+
+def timed_steps(layer, scratch, d, rows, steps, warmup, torch, b1):
+    """W untimed steps, then exactly K steps bracketed by synchronisation; returns ms per step."""
+    def one():
+        b1.ffn_enqueue(layer, scratch, d["payload"].data_ptr(), 4096, d["scales"].data_ptr(), 128, d["ids"].data_ptr(),
+                       d["weights"].data_ptr(), rows, d["out"].data_ptr(), None)
+    for _ in range(warmup):
+        one()
+    scratch.sync()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(steps):
+        one()
+    e1.record()
+    scratch.sync()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    return wall_ms / steps, e0.elapsed_time(e1) / steps
+
+
+def kernel_phases(layer, scratch, d, rows, reps, b1):
+    """Average per-kernel durations from the HIP events the library records on its launch stream."""
+    acc = np.zeros(5)
+    for _ in range(reps):
+        s = b1.ffn_dev(layer, scratch, d["payload"].data_ptr(), 4096, d["scales"].data_ptr(), 128, d["ids"].data_ptr(),
+                       d["weights"].data_ptr(), rows, d["out"].data_ptr(), None)
+        acc += np.array([s.upload_plan_ms, s.phase_ms[0], s.phase_ms[2], s.phase_ms[3], s.gpu_ms])
+    acc /= reps
+    return dict(plan_ms=acc[0], fc1_ms=acc[1], fc2_ms=acc[2], reduce_ms=acc[3], gpu_ms=acc[4])
+
+
+def sample_parity(wl, pools, got_bits, tokens, O):
+    """GPU BF16 rows against the CPU checker on a few tokens."""
+    ref_rc, ref_partial, _, _ = O.layer_ffn(pools, wl.payload[tokens], wl.scales[tokens], wl.ids[tokens], wl.weights[tokens])
+    got = (got_bits[tokens].astype(np.uint32) << 16).view(np.float32).astype(np.float64)
+    ref = ref_partial.astype(np.float64)
+    return dict(tokens=len(tokens), oracle_rc=ref_rc, max_abs_over_max_ref=float(np.max(np.abs(got - ref)) / np.max(np.abs(ref))),
+                mean_rel=float(np.sum(np.abs(got - ref)) / np.sum(np.abs(ref))))
+
+
+def cpu_baseline(wl, pools, tokens, O):
+    """The CPU restatement of the reference's W4A8 expert path on a bounded sample, all host threads."""
+    threads = O.hardware_threads()
+    t0 = time.perf_counter()
+    rc, _, _, _ = O.layer_ffn(pools, wl.payload[tokens], wl.scales[tokens], wl.ids[tokens], wl.weights[tokens], threads=threads)
+    dt = time.perf_counter() - t0
+    return dict(value=len(tokens) / dt, unit="routed tok/s per MoE layer", cores=threads, kind="port",
+                sample=f"{len(tokens)} tokens ({len(tokens) * 8} routes) of the same workload, W4A8 lattice "
+                       f"(FP64 dots, FP32 boundaries), {dt:.1f}s, rc={rc}")
+
+
+def run_config(cfg, steps, warmup, torch, dev, b1, synth, O, parity_tokens, cpu_tokens):
+    wl = synth.make(cfg)
+    log(f"[bench] config {cfg}: {wl.name}")
+    layer, pools = build_layer(wl, torch, dev, b1)
+    scratch = b1.Scratch(stream=torch.cuda.current_stream().cuda_stream)
+    d = stage(wl, torch, dev)
+    ph = kernel_phases(layer, scratch, d, wl.rows, 3, b1)  # also the first correctness pass
+    before = d["out"].cpu().numpy().view(np.uint16).copy()
+    wall_ms, ev_ms = timed_steps(layer, scratch, d, wl.rows, steps, warmup, torch, b1)
+    ph = kernel_phases(layer, scratch, d, wl.rows, 10, b1)
+    after = d["out"].cpu().numpy().view(np.uint16)
+    tokens = np.arange(min(parity_tokens, wl.rows))
+    par = sample_parity(wl, pools, after, tokens, O)
+    par["bitwise_stable_across_timing"] = bool(np.array_equal(before, after))
+    cpu = cpu_baseline(wl, pools, np.arange(min(cpu_tokens, wl.rows)), O) if cpu_tokens else None
+    touched = int(wl.touched().size)
+    res = dict(wl=wl, ms_per_step=wall_ms, event_ms_per_step=ev_ms, phases=ph, parity=par, cpu=cpu, touched=touched)
+    del layer, scratch
+    return res
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--no-prefill", action="store_true", help="skip the 8192-token prefill measurement")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on one GPU only (no collectives, no sharding); use --gpus 1")
+
+    import torch
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible; the HIP path has no CPU fallback")
+    from mimo26f_afd_amd import b1, synth
+    import b1_oracle as O
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+
+    dec = run_config(2, args.steps, args.warmup, torch, dev, b1, synth, O, parity_tokens=8,
+                     cpu_tokens=0 if args.no_cpu else 128)
+    wl = dec["wl"]
+    inter, U = wl.intermediate, dec["touched"]
+    # Algorithmic bytes: unique weight bytes of the touched experts + input rows + ids/weights + BF16 rows;
+    # FC1 streams the gate/up two thirds of each image plus the input rows.
+    path_bytes = wl.algorithmic_bytes()
+    fc1_bytes = U * inter * (4096 + 256) + wl.rows * 4224
+    fc1_gbs = fc1_bytes / (dec["phases"]["fc1_ms"] * 1e-3) / 1e9
+    path_gbs = path_bytes / (dec["ms_per_step"] * 1e-3) / 1e9
+    line = {
+        "metric": "routed tok/s per MoE layer; HBM GB/s (decode) and MFMA % of peak (prefill)",
+        "value": wl.rows / (dec["ms_per_step"] * 1e-3),
+        "unit": "routed tok/s per MoE layer",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": dec["ms_per_step"],
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "fp8xfp4->f32",
+        "data": "synthetic",
+        "config": {"workload": "configs[2]: one full MoE layer, decode/verify, 256 experts x I 2048, H 4096, 128 tokens, top-8",
+                   "experts_touched": U, "routes": wl.rows * 8, "weights": "MXFP4 e2m1 + e8m0/32, uniform codes, scales 2^-8..2^-4",
+                   "activations": "bf16 N(0,1) -> wire quantizer FP8 e4m3 + ue8m0/32"},
+        "roofline": {"bound": "hbm", "kernel": "fc1_kernel<2> (gate/up GEMM + SwiGLU + requant)",
+                     "achieved": fc1_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": fc1_gbs / HBM_PEAK_GBS,
+                     "traffic": None, "algorithmic_bytes": fc1_bytes, "kernel_ms": dec["phases"]["fc1_ms"],
+                     "path": {"algorithmic_bytes": path_bytes, "achieved": path_gbs, "frac": path_gbs / HBM_PEAK_GBS,
+                              "plan_ms": dec["phases"]["plan_ms"], "fc2_ms": dec["phases"]["fc2_ms"],
+                              "reduce_ms": dec["phases"]["reduce_ms"], "event_ms_per_step": dec["event_ms_per_step"]}},
+        "cpu_baseline": dec["cpu"],
+        "parity": dec["parity"],
+    }
+    if not args.no_prefill:
+        pre = run_config(3, max(3, args.steps // 5), max(2, args.warmup // 5), torch, dev, b1, synth, O, parity_tokens=4,
+                         cpu_tokens=0)
+        pw = pre["wl"]
+        flops = pw.flops()
+        tf = flops / (pre["ms_per_step"] * 1e-3) / 1e12
+        fc1_flops = 4 * pw.rows * 8 * 4096 * pw.intermediate
+        fc1_tf = fc1_flops / (pre["phases"]["fc1_ms"] * 1e-3) / 1e12
+        line["prefill"] = {
+            "workload": "configs[3]: one full MoE layer, prefill chunk, 8192 tokens, Zipf(1.1) routing",
+            "value": pw.rows / (pre["ms_per_step"] * 1e-3), "unit": "routed tok/s per MoE layer",
+            "ms_per_step": pre["ms_per_step"], "steps": max(3, args.steps // 5),
+            "roofline": {"bound": "mfma", "kernel": "fc1_kernel<8>", "achieved": fc1_tf, "peak": MFMA_FP8_PEAK_TFLOPS,
+                         "unit": "TFLOP/s", "frac": fc1_tf / MFMA_FP8_PEAK_TFLOPS, "traffic": None,
+                         "algorithmic_flops": fc1_flops, "kernel_ms": pre["phases"]["fc1_ms"],
+                         "path": {"algorithmic_flops": flops, "achieved": tf, "frac": tf / MFMA_FP8_PEAK_TFLOPS,
+                                  "plan_ms": pre["phases"]["plan_ms"], "fc2_ms": pre["phases"]["fc2_ms"],
+                                  "reduce_ms": pre["phases"]["reduce_ms"]}},
+            "parity": pre["parity"],
+        }
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,52 @@
+"""Loads the C-ABI library. There is no fallback: without the HIP library every call raises."""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+from . import build
+
+_u8p, _f32p, _i32p, _u32p, _u16p = (C.POINTER(t) for t in (C.c_uint8, C.c_float, C.c_int32, C.c_uint32, C.c_uint16))
+_vp, _sz, _cp = C.c_void_p, C.c_size_t, C.c_char_p
+
+# name -> (restype, argtypes); every symbol include/m26s_b1.h declares
+SIGNATURES = {
+    "m26s_b1_layer_new": (C.c_int, [_vp, C.c_uint64, C.c_uint32, C.POINTER(_vp), _cp, _sz]),
+    "m26s_b1_layer_all_normal": (C.c_int, [_vp]),
+    "m26s_b1_layer_free": (None, [_vp]),
+    "m26s_b1_scratch_new": (C.c_int, [C.POINTER(_vp), _cp, _sz]),
+    "m26s_b1_scratch_free": (None, [_vp]),
+    "m26s_b1_ffn": (C.c_int, [_vp, _vp, _vp, _sz, _vp, _sz, _vp, _vp, C.c_uint32, _vp, _vp, _cp, _sz]),
+    "m26s_b1_layer_new_full": (C.c_int, [C.POINTER(_vp), C.c_uint64, C.POINTER(_vp), _cp, _sz]),
+    "m26s_b1_layer_intermediate": (C.c_uint32, [_vp]),
+    "m26s_b1_scratch_new_on": (C.c_int, [_vp, C.POINTER(_vp), _cp, _sz]),
+    "m26s_b1_ffn_dev": (C.c_int, [_vp, _vp, _vp, _sz, _vp, _sz, _vp, _vp, C.c_uint32, _vp, _vp, _vp, _cp, _sz]),
+    "m26s_b1_ffn_enqueue": (C.c_int, [_vp, _vp, _vp, _sz, _vp, _sz, _vp, _vp, C.c_uint32, _vp, _vp, _cp, _sz]),
+    "m26s_b1_scratch_sync": (C.c_int, [_vp, _cp, _sz]),
+    "m26s_b1_plan_dev": (C.c_int, [_vp, _vp, C.c_uint32, C.c_uint32, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _cp, _sz]),
+    "m26s_b1_quantize_dev": (C.c_int, [_vp, C.c_uint64, _vp, _vp, _vp, _cp, _sz]),
+    "m26s_b1_reduce_dev": (C.c_int, [_vp, _vp, C.c_uint32, _vp, _vp, _vp, _cp, _sz]),
+    "m26s_b1_scratch_set_taps": (None, [_vp, C.c_int]),
+    "m26s_b1_scratch_view": (C.c_int, [_vp, C.c_int, C.POINTER(_vp), C.POINTER(_sz)]),
+    "m26s_b1_copy_to_host": (C.c_int, [_vp, _vp, _sz]),
+    "m26s_b1_copy_to_device": (C.c_int, [_vp, _vp, _sz]),
+    "m26s_b1_device_alloc": (_vp, [_sz]),
+    "m26s_b1_device_free": (None, [_vp]),
+}
+
+_LIB = None
+
+
+def load() -> C.CDLL:
+    """The built library; built first only if nothing is there."""
+    global _LIB
+    if _LIB is None:
+        if not os.path.exists(build.LIB):
+            build.build_library()
+        lib = C.CDLL(build.LIB)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(lib, name)  # AttributeError here = a declared symbol is not exported
+            fn.restype = res
+            fn.argtypes = args
+        _LIB = lib
+    return _LIB

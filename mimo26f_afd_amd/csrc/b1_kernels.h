@@ -1,0 +1,649 @@
+// gfx950 kernels of the routed-expert FFN (B1, numerical mode E-W4A8-v1).
+//
+// Stage map against the reference (paths relative to the reference repository):
+//   prepare_kernel  <- crates/mimo26-expert/kernels/b1/prepare.cu:39-57 (one-time byte permutation)
+//                      + crates/mimo26-spark/kernels/b1_fc1_m64.cuh:496-512 (scale scan)
+//   plan_kernel     <- crates/mimo26-expert/kernels/b1/group_plan.cu:32-79 (stable plan, the spec)
+//                      + crates/mimo26-spark/kernels/b1_serve.cu:36-96 (one-CTA serving planner, chunks)
+//   fc1_kernel      <- kernels/b1/grouped.cu:74-113 + connected.cu:9-37 (gate/up MMA + SwiGLU)
+//                      fused with kernels/b1/quant_v1.cu:34-68 (intermediate quantizer v1)
+//   fc2_kernel      <- kernels/b1/grouped.cu:135-154 + connected.cu:48-79 (down MMA + inverse scatter)
+//   reduce_kernel   <- kernels/b1/route_reduce.cu:61-124 (weight-once slot-ordered sum, BF16 RNE)
+//   quantize_kernel <- kernels/b1/quant_v1.cu:34-68 (stand-alone form, same device functions)
+#pragma once
+#include <hip/hip_runtime.h>
+#include <float.h>
+#include "b1_layout.h"
+
+namespace m26g {
+
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+struct Canonical {
+    const uint8_t* pool[4];  // ranks x (256 quarter-slice images)
+    uint32_t ranks;          // 1 or 4
+};
+
+struct PlanView {
+    int32_t* inverse;
+    int32_t* original;
+    float* gw;
+    Group* groups;
+    Chunk* chunks;
+    uint32_t* meta;
+};
+
+// ---------------------------------------------------------------------------------------------
+// One-time weight preparation: canonical v2 rank images -> the G950 operand order.
+// grid (any, 256 experts), 256 threads. Pure byte moves; *abnormal is OR-ed with 1 when a weight
+// scale byte lies outside [2, 252].
+// ---------------------------------------------------------------------------------------------
+__global__ void __launch_bounds__(256) prepare_kernel(Canonical c, uint8_t* __restrict__ prepared, Prepared lay,
+                                                      uint32_t* __restrict__ abnormal) {
+    const uint32_t e = blockIdx.y, I = lay.inter;
+    uint8_t* dst = prepared + uint64_t(e) * lay.bytes();
+    const uint64_t img = uint64_t(e) * kImageBytes;
+    const uint32_t stride = gridDim.x * blockDim.x, first = blockIdx.x * blockDim.x + threadIdx.x;
+    bool odd = false;
+    for (uint32_t cell = first; cell < I * 256; cell += stride) {  // w13 payload
+        const uint32_t lane = cell & 63, t = (cell >> 6) & 3, ks = (cell >> 8) & 31, cb = cell >> 13;
+        const uint32_t n = cb * 32 + (t & 1) * 16 + (lane & 15), g = lane >> 4;
+        const uint8_t* src = c.pool[n / kRankI] + img + (t < 2 ? kGatePayload : kUpPayload) +
+                             uint64_t(n % kRankI) * 2048 + ks * 64 + g * 16;
+        *reinterpret_cast<uint4*>(dst + lay.w13() + uint64_t(cell) * 16) = *reinterpret_cast<const uint4*>(src);
+    }
+    for (uint32_t cell = first; cell < I * 64; cell += stride) {  // w13 scales
+        const uint32_t lane = cell & 63, t = (cell >> 6) & 3, q = (cell >> 8) & 7, cb = cell >> 11;
+        const uint32_t n = cb * 32 + (t & 1) * 16 + (lane & 15), g = lane >> 4;
+        const uint8_t* src = c.pool[n / kRankI] + img + (t < 2 ? kGateScales : kUpScales) + uint64_t(n % kRankI) * 128;
+        uint32_t word = 0;
+        for (uint32_t b = 0; b < 4; ++b) {
+            const uint32_t s = src[4 * (4 * q + b) + g];
+            odd = odd || s < 2 || s > 252;
+            word |= s << (8 * b);
+        }
+        *reinterpret_cast<uint32_t*>(dst + lay.s13() + uint64_t(cell) * 4) = word;
+    }
+    const uint32_t ksteps = I / 128, quads = I / 512;
+    for (uint32_t cell = first; cell < I * 128; cell += stride) {  // w2 payload
+        const uint32_t lane = cell & 63, t = (cell >> 6) & 3, ks = (cell >> 8) % ksteps, ob = (cell >> 8) / ksteps;
+        const uint32_t n = ob * 64 + t * 16 + (lane & 15), kb = 4 * ks + (lane >> 4);
+        const uint8_t* src = c.pool[kb / 16] + img + kDownPayload + uint64_t(n) * 256 + (kb % 16) * 16;
+        *reinterpret_cast<uint4*>(dst + lay.w2() + uint64_t(cell) * 16) = *reinterpret_cast<const uint4*>(src);
+    }
+    for (uint32_t cell = first; cell < I * 32; cell += stride) {  // w2 scales
+        const uint32_t lane = cell & 63, t = (cell >> 6) & 3, q = (cell >> 8) % quads, ob = (cell >> 8) / quads;
+        const uint32_t n = ob * 64 + t * 16 + (lane & 15), g = lane >> 4;
+        uint32_t word = 0;
+        for (uint32_t b = 0; b < 4; ++b) {
+            const uint32_t kb = 4 * (4 * q + b) + g;
+            const uint32_t s = c.pool[kb / 16][img + kDownScales + uint64_t(n) * 16 + kb % 16];
+            odd = odd || s < 2 || s > 252;
+            word |= s << (8 * b);
+        }
+        *reinterpret_cast<uint32_t*>(dst + lay.s2() + uint64_t(cell) * 4) = word;
+    }
+    if (odd) atomicOr(abnormal, 1u);
+}
+
+// ---------------------------------------------------------------------------------------------
+// Stage 1: token -> expert bucketing. One workgroup of 1024 threads, LDS counting sort.
+//
+// Bit-exact with the reference's serial planner: routes of one expert keep ascending route order.
+// Each of the 16 waves owns one contiguous run of routes; a wave ranks its 64 routes per step with
+// ballots (no atomics touch a position), per-wave histograms give every wave its start inside each
+// expert, and the second walk places routes. Dynamic LDS holds one id byte per route.
+// ---------------------------------------------------------------------------------------------
+constexpr uint32_t kPlanThreads = 1024, kPlanWaves = kPlanThreads / 64;
+
+__device__ __forceinline__ uint64_t same_expert_lanes(uint32_t e, bool valid) {
+    uint64_t m = __ballot(valid);
+#pragma unroll
+    for (uint32_t b = 0; b < 8; ++b) {
+        const bool bit = (e >> b) & 1u;
+        const uint64_t have = __ballot(bit);
+        m &= bit ? have : ~have;
+    }
+    return m;
+}
+
+// Exclusive scan of 256 values held 4 per lane by one wave; writes base[0..256].
+__device__ __forceinline__ void wave_scan256(const uint32_t (&v)[4], uint32_t* base, uint32_t lane) {
+    const uint32_t total = v[0] + v[1] + v[2] + v[3];
+    uint32_t incl = total;
+#pragma unroll
+    for (uint32_t d = 1; d < 64; d <<= 1) {
+        const uint32_t up = __shfl_up(incl, d);
+        if (lane >= d) incl += up;
+    }
+    uint32_t run = incl - total;
+#pragma unroll
+    for (uint32_t j = 0; j < 4; ++j) {
+        base[4 * lane + j] = run;
+        run += v[j];
+    }
+    if (lane == 63) base[256] = run;
+}
+
+__device__ __forceinline__ uint32_t last_not_above(const uint32_t* base, uint32_t value) {
+    uint32_t lo = 0, hi = 256;  // largest e in [0,256) with base[e] <= value
+    while (hi - lo > 1) {
+        const uint32_t mid = (lo + hi) >> 1;
+        if (base[mid] <= value) lo = mid; else hi = mid;
+    }
+    return lo;
+}
+
+__global__ void __launch_bounds__(kPlanThreads)
+plan_kernel(const int32_t* __restrict__ ids, const float* __restrict__ w, uint32_t rows,
+            const uint8_t* __restrict__ resident, PlanView p, uint32_t gpc, uint32_t reset_capacity) {
+    extern __shared__ uint8_t id_byte[];
+    __shared__ uint32_t hist[kPlanWaves][256];
+    __shared__ uint32_t cnt[256], rbase[257], gbase[257], cbase[257];
+    __shared__ uint32_t first_bad;
+    const uint32_t tid = threadIdx.x, lane = tid & 63, wv = tid >> 6, routes = rows * kTopk;
+
+    for (uint32_t i = tid; i < kPlanWaves * 256; i += kPlanThreads) (&hist[0][0])[i] = 0;
+    if (tid == 0) first_bad = 0xffffffffu;
+    __syncthreads();
+    // Validation keys order faults as the serial planner meets them: (route + 1) << 4 | check,
+    // check 1 = id or residency, 2 = weight, 3 = expert repeated inside the token.
+    if (tid < 256 && resident[tid] > 1) atomicMin(&first_bad, 1u);
+    for (uint32_t i = tid; i < routes; i += kPlanThreads) {
+        const int32_t e = ids[i];
+        const float wt = w[i];
+        uint32_t check = 0;
+        if (e < 0 || e >= int32_t(kExperts) || !resident[e]) check = 1;
+        else if (!(wt >= 0.0f && wt <= FLT_MAX)) check = 2;
+        if (check) atomicMin(&first_bad, ((i + 1) << 4) | check);
+        id_byte[i] = uint8_t(e);
+    }
+    __syncthreads();
+    const uint32_t run = (((routes + kPlanWaves - 1) / kPlanWaves) + 63u) & ~63u;
+    const uint32_t begin = wv * run, end = begin + run < routes ? begin + run : routes;
+    for (uint32_t s = begin; s < end; s += 64) {
+        const uint32_t i = s + lane;
+        const bool valid = i < routes;
+        const uint32_t e = valid ? id_byte[i] : 0;
+        const uint64_t m = same_expert_lanes(e, valid);
+        const uint64_t below = m & ((1ull << lane) - 1);
+        if (valid) {
+            if (below & (0xffull << (lane & ~7u))) atomicMin(&first_bad, ((i + 1) << 4) | 3u);
+            if (!below) hist[wv][e] += __popcll(m);
+        }
+    }
+    __syncthreads();
+    if (first_bad != 0xffffffffu) {
+        if (tid == 0) {
+            const uint32_t check = first_bad & 15u;
+            p.meta[kPlanFault] = check == 2 ? 8u : 7u;  // Status::nonfinite : Status::metadata
+            p.meta[kGroupCount] = 0;
+            p.meta[kChunkCount] = 0;
+        }
+        return;
+    }
+    // The serial planner rewrites every capacity slot once the routes are accepted (inverse /
+    // original = -1, weights = 0, groups = {-1, 0, -1, {-1 x 16}}). Only the stand-alone plan entry
+    // asks for it; the FFN kernels never read past the live counts.
+    for (uint32_t i = tid; i < reset_capacity * 19; i += kPlanThreads) {
+        reinterpret_cast<int32_t*>(p.groups)[i] = (i % 19 == 1) ? 0 : -1;
+        if (i < reset_capacity) {
+            p.inverse[i] = -1;
+            p.original[i] = -1;
+            p.gw[i] = 0.0f;
+        }
+    }
+    if (tid < 256) {
+        uint32_t acc = 0;
+        for (uint32_t k = 0; k < kPlanWaves; ++k) {
+            const uint32_t t = hist[k][tid];
+            hist[k][tid] = acc;
+            acc += t;
+        }
+        cnt[tid] = acc;
+    }
+    __syncthreads();
+    if (wv == 0) {
+        uint32_t a[4], b[4], c[4];
+#pragma unroll
+        for (uint32_t j = 0; j < 4; ++j) {
+            a[j] = cnt[4 * lane + j];
+            b[j] = (a[j] + 15) / 16;
+            c[j] = (b[j] + gpc - 1) / gpc;
+        }
+        wave_scan256(a, rbase, lane);
+        wave_scan256(b, gbase, lane);
+        wave_scan256(c, cbase, lane);
+    }
+    __syncthreads();
+    for (uint32_t s = begin; s < end; s += 64) {
+        const uint32_t i = s + lane;
+        const bool valid = i < routes;
+        const uint32_t e = valid ? id_byte[i] : 0;
+        const uint64_t m = same_expert_lanes(e, valid);
+        const uint64_t below = m & ((1ull << lane) - 1);
+        if (valid) {
+            const uint32_t rel = hist[wv][e] + __popcll(below);
+            const uint32_t pos = rbase[e] + rel;
+            p.original[pos] = int32_t(i);
+            p.inverse[i] = int32_t(pos);
+            p.groups[gbase[e] + rel / 16].input_rows[rel % 16] = int32_t(i / kTopk);
+            if (!below) hist[wv][e] += __popcll(m);
+        }
+    }
+    __syncthreads();
+    for (uint32_t i = tid; i < routes; i += kPlanThreads) p.gw[p.inverse[i]] = w[i];
+    const uint32_t ngroups = gbase[256], nchunks = cbase[256];
+    for (uint32_t gi = tid; gi < ngroups; gi += kPlanThreads) {
+        const uint32_t e = last_not_above(gbase, gi), k = gi - gbase[e];
+        const uint32_t left = cnt[e] - 16 * k, n = left < 16 ? left : 16;
+        Group& G = p.groups[gi];
+        G.expert = int32_t(e);
+        G.rows = int32_t(n);
+        G.route_base = int32_t(rbase[e] + 16 * k);
+        for (uint32_t slot = n; slot < 16; ++slot) G.input_rows[slot] = -1;
+    }
+    for (uint32_t ci = tid; ci < nchunks; ci += kPlanThreads) {
+        const uint32_t e = last_not_above(cbase, ci), j = ci - cbase[e];
+        const uint32_t ng = (cnt[e] + 15) / 16, left = ng - gpc * j;
+        p.chunks[ci] = Chunk{int32_t(gbase[e] + gpc * j), int32_t(left < gpc ? left : gpc)};
+    }
+    if (tid == 0) {
+        p.meta[kGroupCount] = ngroups;
+        p.meta[kChunkCount] = nchunks;
+        p.meta[kPlanFault] = 0;
+    }
+}
+
+// Clears the per-call stage fault words; runs ahead of the planner on the same stream.
+__global__ void meta_reset_kernel(uint32_t* meta) {
+    if (threadIdx.x < kMetaWords) meta[threadIdx.x] = threadIdx.x == kQuantWhere ? 0xffffffffu : 0u;
+}
+
+// ---------------------------------------------------------------------------------------------
+// Intermediate quantizer v1 on FP32 bit patterns (byte-exact contract):
+// crates/mimo26-expert/kernels/b1/quant_v1.cuh:32-100, oracle/lattice/quant_v1.py:74-87.
+// ---------------------------------------------------------------------------------------------
+constexpr uint32_t kQuantFloorBits = 0x38d1b717u;  // FP32(1e-4)
+
+// k = smallest integer with amax <= 448 * 2^k, amax already floored (so it is a normal number).
+__device__ __forceinline__ int quant_scale_exponent(uint32_t amax_bits) {
+    const uint32_t a = amax_bits < kQuantFloorBits ? kQuantFloorBits : amax_bits;
+    return int(a >> 23) - 127 - ((a & 0x7fffffu) <= 0x600000u ? 8 : 7);
+}
+
+// Round-half-even of value / 2^shift for value < 2^24, shift >= 1.
+__device__ __forceinline__ uint32_t rne_shift(uint32_t value, int shift) {
+    if (shift > 25) return 0;
+    const uint32_t q = value >> shift, rem = value & ((1u << shift) - 1u), half = 1u << (shift - 1);
+    return q + ((rem > half || (rem == half && (q & 1u))) ? 1u : 0u);
+}
+
+// E4M3FN code of h * 2^-k, ties to even, sign of zero kept.
+__device__ __forceinline__ uint32_t quant_code(uint32_t bits, int k) {
+    const uint32_t sign = (bits >> 24) & 0x80u, mag = bits & 0x7fffffffu;
+    if (!mag) return sign;
+    const uint32_t field = mag >> 23;
+    // A subnormal input is far below the floor-derived quantum: it rounds to zero for every legal k.
+    if (!field) return sign;
+    const uint32_t sig = (mag & 0x7fffffu) | 0x800000u;
+    int e = int(field) - 127 - k;
+    uint32_t code;
+    if (e < -6) {
+        code = rne_shift(sig, 14 - e);  // quantum 2^-9; a carry into 8 is the first normal code
+    } else {
+        uint32_t r = rne_shift(sig, 20);
+        if (r == 16) { r = 8; ++e; }
+        code = uint32_t(e + 7) * 8 + r - 8;
+        if (code > 126) code = 126;
+    }
+    return sign | code;
+}
+
+__device__ __forceinline__ bool quant_reconstructs(uint32_t code, int k) {
+    const uint32_t field = (code & 0x7fu) >> 3;
+    return field == 0 || int(field) - 7 + k <= 127;
+}
+
+// Stand-alone quantizer: one K32 block per half-wave (two blocks per wave per step).
+__global__ void __launch_bounds__(256) quantize_kernel(const float* __restrict__ h, uint64_t blocks,
+                                                       uint8_t* __restrict__ payload, uint8_t* __restrict__ scales,
+                                                       uint32_t* __restrict__ faults) {
+    const uint32_t sub = threadIdx.x & 31;
+    const uint64_t first = (uint64_t(blockIdx.x) * blockDim.x + threadIdx.x) >> 5;
+    const uint64_t stride = (uint64_t(gridDim.x) * blockDim.x) >> 5;
+    for (uint64_t b = first; b < blocks; b += stride) {
+        const uint32_t bits = __float_as_uint(h[b * 32 + sub]);
+        uint32_t amax = bits & 0x7fffffffu;
+#pragma unroll
+        for (int d = 16; d; d >>= 1) {
+            const uint32_t o = __shfl_xor(amax, d);
+            amax = o > amax ? o : amax;
+        }
+        if (amax >= 0x7f800000u) {
+            if (sub == 0) faults[b] = 1;
+            continue;
+        }
+        const int k = quant_scale_exponent(amax);
+        const uint32_t code = quant_code(bits, k);
+        uint32_t over = quant_reconstructs(code, k) ? 0u : 1u;
+#pragma unroll
+        for (int d = 16; d; d >>= 1) over |= __shfl_xor(over, d);
+        if (sub == 0) faults[b] = over ? 2u : 0u;
+        if (over) continue;
+        payload[b * 32 + sub] = uint8_t(code);
+        if (sub == 0) scales[b] = uint8_t(k + 127);
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Block-scaled grouped GEMM core, shared by FC1 and FC2.
+//
+// One wave owns four 16-row weight tiles (SrcA, FP4, streamed once, fully coalesced 1 KB per
+// tile per k-step) and up to NT 16-row activation tiles (SrcB, FP8, row-major rows gathered by
+// pointer). A k-step is K = 128. Loads for step k+1 are issued before the MFMAs of step k.
+// ---------------------------------------------------------------------------------------------
+template <int NT>
+struct Operands {
+    v4i a[4];
+    v4i lo[NT], hi[NT];
+    uint32_t sb[NT];
+};
+
+template <int NT>
+__device__ __forceinline__ void load_step(Operands<NT>& o, const uint8_t* __restrict__ wp, int ks,
+                                          const uint8_t* const (&xrow)[NT], const uint8_t* const (&xsrow)[NT],
+                                          int tiles) {
+#pragma unroll
+    for (int t = 0; t < 4; ++t) o.a[t] = *reinterpret_cast<const v4i*>(wp + size_t(ks) * 4096 + t * 1024);
+#pragma unroll
+    for (int tt = 0; tt < NT; ++tt)
+        if (tt < tiles) {
+            o.lo[tt] = *reinterpret_cast<const v4i*>(xrow[tt] + ks * 128);
+            o.hi[tt] = *reinterpret_cast<const v4i*>(xrow[tt] + ks * 128 + 64);
+            o.sb[tt] = *reinterpret_cast<const uint32_t*>(xsrow[tt] + ks * 4);
+        }
+}
+
+template <int NT, int SEL>
+__device__ __forceinline__ void mfma_step(v4f (&acc)[4][NT], const Operands<NT>& o, const uint32_t (&sw)[4],
+                                          int tiles, uint32_t shift, uint32_t& bad) {
+#pragma unroll
+    for (int tt = 0; tt < NT; ++tt)
+        if (tt < tiles) {
+            const uint32_t s = (o.sb[tt] >> shift) & 0xffu;
+            bad |= (s - 105u) > 142u ? 1u : 0u;  // activation scales are legal only in [105, 247]
+            const v8i b = {o.lo[tt].x, o.lo[tt].y, o.lo[tt].z, o.lo[tt].w, o.hi[tt].x, o.hi[tt].y, o.hi[tt].z, o.hi[tt].w};
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                const v8i a = {o.a[t].x, o.a[t].y, o.a[t].z, o.a[t].w, 0, 0, 0, 0};
+                acc[t][tt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, acc[t][tt], 4 /*A: E2M1*/,
+                                                                              0 /*B: E4M3*/, SEL, int(sw[t]), 0, int(s));
+            }
+        }
+}
+
+// wp / sp already include the lane offset (lane*16, lane*4). ksteps is a multiple of 4.
+template <int NT>
+__device__ __forceinline__ void gemm_chunk(v4f (&acc)[4][NT], const uint8_t* __restrict__ wp,
+                                           const uint8_t* __restrict__ sp, int ksteps,
+                                           const uint8_t* const (&xrow)[NT], const uint8_t* const (&xsrow)[NT],
+                                           int tiles, uint32_t lane, uint32_t& bad) {
+    const uint32_t shift = 8 * (lane >> 4);
+    Operands<NT> cur, nxt;
+    load_step<NT>(cur, wp, 0, xrow, xsrow, tiles);
+    for (int q = 0; q < ksteps / 4; ++q) {
+        uint32_t sw[4];
+#pragma unroll
+        for (int t = 0; t < 4; ++t) sw[t] = *reinterpret_cast<const uint32_t*>(sp + size_t(q) * 1024 + t * 256);
+        const int ks = 4 * q;
+        load_step<NT>(nxt, wp, ks + 1, xrow, xsrow, tiles);
+        mfma_step<NT, 0>(acc, cur, sw, tiles, shift, bad);
+        load_step<NT>(cur, wp, ks + 2, xrow, xsrow, tiles);
+        mfma_step<NT, 1>(acc, nxt, sw, tiles, shift, bad);
+        load_step<NT>(nxt, wp, ks + 3, xrow, xsrow, tiles);
+        mfma_step<NT, 2>(acc, cur, sw, tiles, shift, bad);
+        if (ks + 4 < ksteps) load_step<NT>(cur, wp, ks + 4, xrow, xsrow, tiles);
+        mfma_step<NT, 3>(acc, nxt, sw, tiles, shift, bad);
+    }
+}
+
+// SwiGLU in the reference's stable form (kernels/b1/grouped.cu:89-93) with the CPU reference's
+// exponential: binary64 exp rounded once to binary32 (mimo26-repack/tests/lattice_oracle.py:32-53).
+__device__ __forceinline__ float silu_up(float g, float u) {
+    const float t = g >= 0.0f ? -g : g;
+    const float e = float(exp(double(t)));
+    const float d = __fadd_rn(1.0f, e);
+    const float s = g >= 0.0f ? __fdiv_rn(g, d) : __fdiv_rn(__fmul_rn(g, e), d);
+    return __fmul_rn(s, u);
+}
+
+struct Fc1Args {
+    const uint8_t* prepared;
+    Prepared lay;
+    PlanView plan;
+    const uint8_t* x;         // E4M3 rows
+    size_t x_pitch;
+    const uint8_t* xs;        // UE8M0 K32 scale rows
+    size_t xs_pitch;
+    const uint8_t* zero_row;  // >= 4096 + 64 zero bytes, stands in for padded rows
+    const uint8_t* unit_scales;  // >= 128 bytes of 127
+    uint8_t* dq;              // [groups*16][I] E4M3 intermediate
+    uint8_t* dqs;             // [groups*16][I/32] its scales
+    float* tap_gate;          // optional FP32 taps [groups*16][I]
+    float* tap_up;
+    float* tap_h;
+};
+
+// Stages 2+3: gate/up grouped GEMM, SwiGLU and the v1 requantisation of the intermediate.
+// grid (I/128, chunk capacity), 256 threads; each wave owns one 32-column K32 block of the
+// intermediate for every row of its chunk, so a quantizer block never leaves the wave.
+template <int NT>
+__global__ void __launch_bounds__(256) fc1_kernel(Fc1Args a) {
+    uint32_t* meta = a.plan.meta;
+    const uint32_t c = blockIdx.y;
+    if (meta[kPlanFault] || c >= meta[kChunkCount]) return;
+    const Chunk ch = a.plan.chunks[c];
+    const uint32_t lane = threadIdx.x & 63, wv = threadIdx.x >> 6, r = lane & 15, g = lane >> 4;
+    const uint32_t I = a.lay.inter, cb = blockIdx.x * 4 + wv;
+    const int tiles = ch.groups < NT ? ch.groups : NT;
+    const Group* grp = a.plan.groups + ch.first_group;
+    const int32_t expert = grp[0].expert;
+    if (expert < 0 || expert >= int32_t(kExperts) || tiles < 1) {
+        if (lane == 0) atomicOr(&meta[kFc1Fault], 2u);
+        return;
+    }
+    const uint8_t* xrow[NT];
+    const uint8_t* xsrow[NT];
+    bool live[NT];
+#pragma unroll
+    for (int tt = 0; tt < NT; ++tt) {
+        const int32_t row = tt < tiles ? grp[tt].input_rows[r] : -1;
+        live[tt] = row >= 0;
+        xrow[tt] = (live[tt] ? a.x + size_t(row) * a.x_pitch : a.zero_row) + g * 16;
+        xsrow[tt] = live[tt] ? a.xs + size_t(row) * a.xs_pitch : a.unit_scales;
+    }
+    const uint8_t* img = a.prepared + uint64_t(expert) * a.lay.bytes();
+    const uint8_t* wp = img + a.lay.w13() + uint64_t(cb) * (32 * 4096) + lane * 16;
+    const uint8_t* sp = img + a.lay.s13() + uint64_t(cb) * (8 * 1024) + lane * 4;
+    v4f acc[4][NT];
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+        for (int tt = 0; tt < NT; ++tt) acc[t][tt] = v4f{0.f, 0.f, 0.f, 0.f};
+    uint32_t bad = 0;
+    gemm_chunk<NT>(acc, wp, sp, 32, xrow, xsrow, tiles, lane, bad);
+    bad |= __shfl_xor(bad, 16);
+    bad |= __shfl_xor(bad, 32);
+
+#pragma unroll
+    for (int tt = 0; tt < NT; ++tt) {
+        if (tt >= tiles) continue;
+        float h[2][4];
+        uint32_t amax = 0;
+#pragma unroll
+        for (int t2 = 0; t2 < 2; ++t2)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                h[t2][i] = silu_up(acc[t2][tt][i], acc[t2 + 2][tt][i]);
+                const uint32_t m = __float_as_uint(h[t2][i]) & 0x7fffffffu;
+                amax = m > amax ? m : amax;
+            }
+        uint32_t o = __shfl_xor(amax, 16);
+        amax = o > amax ? o : amax;
+        o = __shfl_xor(amax, 32);
+        amax = o > amax ? o : amax;
+        const size_t grow = size_t(ch.first_group + tt) * 16 + r;
+        const size_t col = size_t(cb) * 32 + 4 * g;
+        if (live[tt] && a.tap_h) {
+#pragma unroll
+            for (int t2 = 0; t2 < 2; ++t2) {
+                *reinterpret_cast<v4f*>(a.tap_gate + grow * I + col + 16 * t2) = acc[t2][tt];
+                *reinterpret_cast<v4f*>(a.tap_up + grow * I + col + 16 * t2) = acc[t2 + 2][tt];
+                *reinterpret_cast<v4f*>(a.tap_h + grow * I + col + 16 * t2) = v4f{h[t2][0], h[t2][1], h[t2][2], h[t2][3]};
+            }
+        }
+        const uint32_t block = uint32_t(grow * (I / 32) + cb);
+        uint32_t fault = (amax >= 0x7f800000u || bad) ? 1u : 0u;
+        const int k = quant_scale_exponent(amax);
+        uint32_t word[2] = {0, 0};
+        if (!fault) {
+            uint32_t over = 0;
+#pragma unroll
+            for (int t2 = 0; t2 < 2; ++t2)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const uint32_t code = quant_code(__float_as_uint(h[t2][i]), k);
+                    over |= quant_reconstructs(code, k) ? 0u : 1u;
+                    word[t2] |= code << (8 * i);
+                }
+            over |= __shfl_xor(over, 16);
+            over |= __shfl_xor(over, 32);
+            if (over) fault = 2;
+        }
+        if (!live[tt]) continue;
+        if (fault) {
+            if (g == 0) {
+                atomicOr(&meta[kQuantFault], fault);
+                atomicMin(&meta[kQuantWhere], block);
+            }
+            continue;  // a faulting block publishes no bytes
+        }
+        *reinterpret_cast<uint32_t*>(a.dq + grow * I + col) = word[0];
+        *reinterpret_cast<uint32_t*>(a.dq + grow * I + col + 16) = word[1];
+        if (g == 0) a.dqs[grow * (I / 32) + cb] = uint8_t(k + 127);
+    }
+}
+
+struct Fc2Args {
+    const uint8_t* prepared;
+    Prepared lay;
+    PlanView plan;
+    const uint8_t* dq;
+    const uint8_t* dqs;
+    const uint8_t* zero_row;
+    const uint8_t* unit_scales;
+    float* y;         // [routes][4096], original (token, slot) order, unweighted
+    uint32_t routes;
+};
+
+// Stage 4a: down grouped GEMM on the requantised intermediate; rows go back to y[original route].
+// grid (16, chunk capacity), 256 threads; each wave owns 64 output columns.
+template <int NT>
+__global__ void __launch_bounds__(256) fc2_kernel(Fc2Args a) {
+    uint32_t* meta = a.plan.meta;
+    const uint32_t c = blockIdx.y;
+    if (meta[kPlanFault] || meta[kFc1Fault] || meta[kQuantFault] || c >= meta[kChunkCount]) return;
+    const Chunk ch = a.plan.chunks[c];
+    const uint32_t lane = threadIdx.x & 63, wv = threadIdx.x >> 6, r = lane & 15, g = lane >> 4;
+    const uint32_t I = a.lay.inter, ob = blockIdx.x * 4 + wv;
+    const int tiles = ch.groups < NT ? ch.groups : NT;
+    const Group* grp = a.plan.groups + ch.first_group;
+    const int32_t expert = grp[0].expert;
+    if (expert < 0 || expert >= int32_t(kExperts) || tiles < 1) {
+        if (lane == 0) atomicOr(&meta[kFc2Fault], 2u);
+        return;
+    }
+    const uint8_t* xrow[NT];
+    const uint8_t* xsrow[NT];
+    int32_t route[NT];
+#pragma unroll
+    for (int tt = 0; tt < NT; ++tt) {
+        const bool live = tt < tiles && int32_t(r) < grp[tt].rows;
+        const size_t grow = size_t(ch.first_group + tt) * 16 + r;
+        route[tt] = live ? a.plan.original[grp[tt].route_base + r] : -1;
+        xrow[tt] = (live ? a.dq + grow * I : a.zero_row) + g * 16;
+        xsrow[tt] = live ? a.dqs + grow * (I / 32) : a.unit_scales;
+    }
+    const uint32_t ksteps = I / 128;
+    const uint8_t* img = a.prepared + uint64_t(expert) * a.lay.bytes();
+    const uint8_t* wp = img + a.lay.w2() + uint64_t(ob) * ksteps * 4096 + lane * 16;
+    const uint8_t* sp = img + a.lay.s2() + uint64_t(ob) * (ksteps / 4) * 1024 + lane * 4;
+    v4f acc[4][NT];
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+        for (int tt = 0; tt < NT; ++tt) acc[t][tt] = v4f{0.f, 0.f, 0.f, 0.f};
+    uint32_t bad = 0;
+    gemm_chunk<NT>(acc, wp, sp, int(ksteps), xrow, xsrow, tiles, lane, bad);
+    bool lost = false;
+#pragma unroll
+    for (int tt = 0; tt < NT; ++tt) {
+        if (tt >= tiles || route[tt] < 0) continue;
+        if (uint32_t(route[tt]) >= a.routes) { lost = true; continue; }
+        float* dst = a.y + size_t(route[tt]) * kHidden + ob * 64 + 4 * g;
+#pragma unroll
+        for (int t = 0; t < 4; ++t) *reinterpret_cast<v4f*>(dst + 16 * t) = acc[t][tt];
+    }
+    if (lost) atomicOr(&meta[kFc2Fault], 5u);
+}
+
+// Stage 4b: router-weighted combine. Per (token, column): v = 0; for slot 0..7:
+// v = RN(v + RN(w * z)) with two roundings; BF16 RNE; nonfinite or negative inputs, a nonfinite
+// running sum or a BF16 exponent of all ones raise the fault word. Four columns per thread.
+__global__ void __launch_bounds__(256) reduce_kernel(const float* __restrict__ y, const float* __restrict__ w,
+                                                     uint32_t rows, float* __restrict__ partial,
+                                                     uint16_t* __restrict__ bf16, uint32_t* __restrict__ fault,
+                                                     const uint32_t* __restrict__ gate) {
+    if (gate && (gate[kPlanFault] || gate[kFc1Fault] || gate[kQuantFault] || gate[kFc2Fault])) return;
+    const uint64_t n4 = uint64_t(rows) * (kHidden / 4);
+    bool failed = false;
+    for (uint64_t i = uint64_t(blockIdx.x) * blockDim.x + threadIdx.x; i < n4; i += uint64_t(gridDim.x) * blockDim.x) {
+        const uint64_t row = i / (kHidden / 4), col = (i % (kHidden / 4)) * 4;
+        v4f z[8];
+#pragma unroll
+        for (int s = 0; s < 8; ++s) z[s] = *reinterpret_cast<const v4f*>(y + (row * 8 + s) * kHidden + col);
+        float v[4] = {0.f, 0.f, 0.f, 0.f};
+        bool ok = true;
+#pragma unroll
+        for (int s = 0; s < 8; ++s) {
+            const float wt = w[row * 8 + s];
+            ok = ok && wt >= 0.0f && wt <= FLT_MAX;
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                ok = ok && fabsf(z[s][k]) <= FLT_MAX;
+                v[k] = __fadd_rn(v[k], __fmul_rn(wt, z[s][k]));
+                ok = ok && fabsf(v[k]) <= FLT_MAX;
+            }
+        }
+        uint32_t code[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const uint32_t b = __float_as_uint(v[k]);
+            code[k] = (b + 0x7fffu + ((b >> 16) & 1u)) >> 16;
+            ok = ok && (code[k] & 0x7f80u) != 0x7f80u;
+        }
+        if (!ok) {
+            failed = true;
+            v[0] = v[1] = v[2] = v[3] = __uint_as_float(0x7fc00000u);
+            code[0] = code[1] = code[2] = code[3] = 0;
+        }
+        if (partial) *reinterpret_cast<v4f*>(partial + row * kHidden + col) = v4f{v[0], v[1], v[2], v[3]};
+        *reinterpret_cast<uint2*>(bf16 + row * kHidden + col) = make_uint2(code[0] | (code[1] << 16), code[2] | (code[3] << 16));
+    }
+    if (failed) atomicOr(fault, 8u);  // Status::nonfinite
+}
+
+}  // namespace m26g

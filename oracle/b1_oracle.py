@@ -1,0 +1,251 @@
+"""ctypes binding of the CPU checker (oracle/liboracle.so) and, where it was built, of the
+reference's own B1 host units (oracle/_ref/libb1ref.so).
+
+TEST INFRASTRUCTURE ONLY: imported by tests/, the smoke check and the benchmark's
+cpu_baseline leg; never by the product package.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+HIDDEN, EXPERTS, TOPK, RANK_I, IMAGE_BYTES = 4096, 256, 8, 512, 3342336
+GROUP_DTYPE = np.dtype([("expert", "<i4"), ("rows", "<i4"), ("route_base", "<i4"), ("input_rows", "<i4", (16,))])
+assert GROUP_DTYPE.itemsize == 76
+
+_u8p, _f32p, _i32p, _u32p, _u16p = (C.POINTER(t) for t in (C.c_uint8, C.c_float, C.c_int32, C.c_uint32, C.c_uint16))
+
+
+def build(force: bool = False) -> None:
+    """Compile the checker (and the reference units when /root/reference is present)."""
+    if force or not os.path.exists(os.path.join(HERE, "liboracle.so")):
+        subprocess.run(["make", "-C", HERE, "-B" if force else "-s", "all"], check=True)
+
+
+def _p(a, t):
+    return a.ctypes.data_as(t) if a is not None else None
+
+
+class _Layer(C.Structure):
+    _fields_ = [("pool", C.c_void_p * 4), ("ranks", C.c_uint32)]
+
+
+def _load():
+    build()
+    lib = C.CDLL(os.path.join(HERE, "liboracle.so"))
+    lib.orc_mxfp4_bits.restype = C.c_uint32
+    lib.orc_mxfp4_bits.argtypes = [C.c_uint32, C.c_uint32]
+    lib.orc_e4m3_value.restype = C.c_float
+    lib.orc_e4m3_value.argtypes = [C.c_uint8]
+    lib.orc_bf16_rne.restype = C.c_uint16
+    lib.orc_bf16_rne.argtypes = [C.c_float]
+    lib.orc_e4m3_encode_half_up.restype = C.c_uint8
+    lib.orc_e4m3_encode_half_up.argtypes = [C.c_double]
+    lib.orc_silu_up.restype = C.c_float
+    lib.orc_silu_up.argtypes = [C.c_float, C.c_float]
+    lib.orc_quant_v1.restype = C.c_size_t
+    lib.orc_activation_decode.restype = C.c_size_t
+    lib.orc_plan.restype = C.c_uint32
+    lib.orc_reduce.restype = C.c_uint32
+    lib.orc_expert_ffn.restype = C.c_uint32
+    lib.orc_layer_ffn.restype = C.c_uint32
+    lib.orc_layer_ffn_efp32.restype = C.c_uint32
+    lib.orc_hardware_threads.restype = C.c_int
+    return lib
+
+
+LIB = _load()
+
+
+def hardware_threads() -> int:
+    return int(LIB.orc_hardware_threads())
+
+
+def mxfp4_bits(nibble: int, scale: int) -> int:
+    return int(LIB.orc_mxfp4_bits(nibble, scale))
+
+
+def mxfp4_rows(payload: np.ndarray, scales: np.ndarray) -> np.ndarray:
+    """payload u8 [n, k/2], scales u8 [n, k/32] -> f32 [n, k]."""
+    payload = np.ascontiguousarray(payload, np.uint8)
+    scales = np.ascontiguousarray(scales, np.uint8)
+    n, half = payload.shape
+    out = np.empty((n, half * 2), np.float32)
+    for r in range(n):
+        LIB.orc_mxfp4_row(_p(payload[r], _u8p), _p(scales[r], _u8p), C.c_size_t(half * 2), _p(out[r], _f32p))
+    return out
+
+
+def e4m3_value(code: int) -> float:
+    return float(LIB.orc_e4m3_value(code))
+
+
+def activation_decode(payload: np.ndarray, scales: np.ndarray):
+    payload = np.ascontiguousarray(payload, np.uint8)
+    scales = np.ascontiguousarray(scales, np.uint8)
+    rows, cols = payload.shape
+    out = np.empty((rows, cols), np.float32)
+    bad = LIB.orc_activation_decode(_p(payload, _u8p), C.c_size_t(cols), _p(scales, _u8p), C.c_size_t(cols // 32),
+                                    C.c_size_t(rows), C.c_size_t(cols), _p(out, _f32p))
+    return out, int(bad)
+
+
+def q0_quantize(x: np.ndarray):
+    x = np.ascontiguousarray(x, np.float32)
+    rows, cols = x.shape
+    payload = np.empty((rows, cols), np.uint8)
+    scales = np.empty((rows, cols // 32), np.uint8)
+    LIB.orc_q0_quantize(_p(x, _f32p), C.c_size_t(rows), C.c_size_t(cols), _p(payload, _u8p), _p(scales, _u8p))
+    return payload, scales
+
+
+def quant_v1(h: np.ndarray, fill: int = 0xA5):
+    """f32 [..., n] -> (payload, scales, faults); faulting blocks keep the fill byte."""
+    h = np.ascontiguousarray(h, np.float32)
+    n = h.size
+    payload = np.full(h.shape, fill, np.uint8)
+    scales = np.full(h.shape[:-1] + (h.shape[-1] // 32,), fill, np.uint8)
+    faults = np.zeros(n // 32, np.uint32)
+    LIB.orc_quant_v1(_p(h, _f32p), C.c_size_t(n), _p(payload, _u8p), _p(scales, _u8p), _p(faults, _u32p))
+    return payload, scales, faults.reshape(scales.shape)
+
+
+class Plan:
+    def __init__(self, capacity: int):
+        n = capacity * 8
+        self.inverse = np.full(n, 0x5A5A5A5A, np.int32)
+        self.original_routes = np.full(n, 0x5A5A5A5A, np.int32)
+        self.grouped_weights = np.full(n, 123.0, np.float32)
+        self.groups = np.zeros(n, GROUP_DTYPE)
+        self.groups["expert"] = 0x5A5A5A5A
+        self.group_count = np.full(1, 0x5A5A5A5A, np.uint32)
+        self.fault = np.full(1, 0x5A5A5A5A, np.uint32)
+        self.status = None
+
+
+def _plan_call(fn, capacity, ids, weights, resident, out: Plan):
+    ids = np.ascontiguousarray(ids, np.int32).reshape(-1)
+    weights = np.ascontiguousarray(weights, np.float32).reshape(-1)
+    rows = ids.size // 8
+    if resident is None:
+        resident = np.ones(256, np.uint8)
+    resident = np.ascontiguousarray(resident, np.uint8)
+    out.status = int(fn(C.c_uint32(capacity), C.c_uint32(rows), _p(ids, _i32p), _p(weights, _f32p), _p(resident, _u8p),
+                        _p(out.inverse, _i32p), _p(out.original_routes, _i32p), _p(out.grouped_weights, _f32p),
+                        out.groups.ctypes.data_as(C.c_void_p), _p(out.group_count, _u32p), _p(out.fault, _u32p)))
+    return out
+
+
+def plan(capacity, ids, weights, resident=None, out: Plan | None = None) -> Plan:
+    return _plan_call(LIB.orc_plan, capacity, ids, weights, resident, out or Plan(capacity))
+
+
+def silu_up(g, u) -> np.ndarray:
+    g = np.asarray(g, np.float32)
+    u = np.asarray(u, np.float32)
+    return np.array([LIB.orc_silu_up(float(a), float(b)) for a, b in zip(g.reshape(-1), u.reshape(-1))],
+                    np.float32).reshape(g.shape)
+
+
+def reduce(y: np.ndarray, w: np.ndarray):
+    """y f32 [rows, 8, cols], w f32 [rows, 8] -> (status, partial f32 [rows, cols], bf16 u16)."""
+    y = np.ascontiguousarray(y, np.float32)
+    w = np.ascontiguousarray(w, np.float32)
+    rows, _, cols = y.shape
+    partial = np.zeros((rows, cols), np.float32)
+    bf16 = np.zeros((rows, cols), np.uint16)
+    st = LIB.orc_reduce(_p(y, _f32p), _p(w, _f32p), C.c_size_t(rows), C.c_size_t(cols), _p(partial, _f32p), _p(bf16, _u16p))
+    return int(st), partial, bf16
+
+
+def _layer(pools) -> _Layer:
+    L = _Layer()
+    for i, p in enumerate(pools):
+        assert p.dtype == np.uint8 and p.flags.c_contiguous and p.size == EXPERTS * IMAGE_BYTES
+        L.pool[i] = p.ctypes.data
+    L.ranks = len(pools)
+    return L
+
+
+def expert_ffn(pools, expert: int, x_payload: np.ndarray, x_scales: np.ndarray):
+    """One expert over the given activation rows. Returns a dict of every stage."""
+    xp = np.ascontiguousarray(x_payload, np.uint8)
+    xs = np.ascontiguousarray(x_scales, np.uint8)
+    rows = xp.shape[0]
+    inter = RANK_I * len(pools)
+    out = dict(gate=np.zeros((rows, inter), np.float32), up=np.zeros((rows, inter), np.float32),
+               h=np.zeros((rows, inter), np.float32), mid_payload=np.zeros((rows, inter), np.uint8),
+               mid_scales=np.zeros((rows, inter // 32), np.uint8), y=np.zeros((rows, HIDDEN), np.float32))
+    L = _layer(pools)
+    out["fault"] = int(LIB.orc_expert_ffn(C.byref(L), C.c_uint32(expert), _p(xp, _u8p), C.c_size_t(xp.shape[1]),
+                                          _p(xs, _u8p), C.c_size_t(xs.shape[1]), C.c_size_t(rows),
+                                          _p(out["gate"], _f32p), _p(out["up"], _f32p), _p(out["h"], _f32p),
+                                          _p(out["mid_payload"], _u8p), _p(out["mid_scales"], _u8p), _p(out["y"], _f32p)))
+    return out
+
+
+def layer_ffn(pools, x_payload, x_scales, ids, weights, threads: int = 0, want_routes: bool = False, efp32: bool = False):
+    """Whole layer. Returns (rc, partial f32 [rows,4096], bf16 u16 [rows,4096], y_routes or None)."""
+    xp = np.ascontiguousarray(x_payload, np.uint8)
+    xs = np.ascontiguousarray(x_scales, np.uint8)
+    ids = np.ascontiguousarray(ids, np.int32).reshape(-1)
+    weights = np.ascontiguousarray(weights, np.float32).reshape(-1)
+    rows = xp.shape[0]
+    partial = np.zeros((rows, HIDDEN), np.float32)
+    bf16 = np.zeros((rows, HIDDEN), np.uint16)
+    L = _layer(pools)
+    if efp32:
+        rc = LIB.orc_layer_ffn_efp32(C.byref(L), _p(xp, _u8p), C.c_size_t(xp.shape[1]), _p(xs, _u8p), C.c_size_t(xs.shape[1]),
+                                     _p(ids, _i32p), _p(weights, _f32p), C.c_size_t(rows), _p(partial, _f32p),
+                                     _p(bf16, _u16p), C.c_int(threads))
+        return int(rc), partial, bf16, None
+    yr = np.zeros((rows * 8, HIDDEN), np.float32) if want_routes else None
+    rc = LIB.orc_layer_ffn(C.byref(L), _p(xp, _u8p), C.c_size_t(xp.shape[1]), _p(xs, _u8p), C.c_size_t(xs.shape[1]),
+                           _p(ids, _i32p), _p(weights, _f32p), C.c_size_t(rows), _p(yr, _f32p), _p(partial, _f32p),
+                           _p(bf16, _u16p), C.c_int(threads))
+    return int(rc), partial, bf16, yr
+
+
+# ---- the reference's own host units, where built (differential checks only) -------------------
+def _load_ref():
+    path = os.path.join(HERE, "_ref", "libb1ref.so")
+    if not os.path.exists(path):
+        return None
+    lib = C.CDLL(path)
+    lib.ref_mxfp4_bits.restype = C.c_uint32
+    lib.ref_mxfp4_bits.argtypes = [C.c_uint32, C.c_uint32]
+    for f in (lib.ref_quant_v1, lib.ref_plan, lib.ref_reduce):
+        f.restype = C.c_uint32
+    return lib
+
+
+REF = _load_ref()
+
+
+def ref_quant_v1(h: np.ndarray, fill: int = 0xA5):
+    h = np.ascontiguousarray(h, np.float32)
+    n = h.size
+    payload = np.full(h.shape, fill, np.uint8)
+    scales = np.full(h.shape[:-1] + (h.shape[-1] // 32,), fill, np.uint8)
+    faults = np.zeros(n // 32, np.uint32)
+    st = REF.ref_quant_v1(_p(h, _f32p), C.c_uint64(n), _p(payload, _u8p), _p(scales, _u8p), _p(faults, _u32p))
+    return payload, scales, faults.reshape(scales.shape), int(st)
+
+
+def ref_plan(capacity, ids, weights, resident=None, out: Plan | None = None) -> Plan:
+    return _plan_call(REF.ref_plan, capacity, ids, weights, resident, out or Plan(capacity))
+
+
+def ref_reduce(y: np.ndarray, w: np.ndarray):
+    y = np.ascontiguousarray(y, np.float32)
+    w = np.ascontiguousarray(w, np.float32)
+    rows = y.shape[0]
+    partial = np.zeros((rows, HIDDEN), np.float32)
+    bf16 = np.zeros((rows, HIDDEN), np.uint16)
+    fault = np.zeros(1, np.uint32)
+    st = REF.ref_reduce(_p(y, _f32p), _p(w, _f32p), C.c_uint32(rows), _p(partial, _f32p), _p(bf16, _u16p), _p(fault, _u32p))
+    return int(st), partial, bf16

@@ -1,0 +1,49 @@
+"""Shared pieces of the GPU parity tests: device staging through the library's own helpers and the
+parity metrics the benchmark contract states."""
+from __future__ import annotations
+
+import numpy as np
+
+from mimo26f_afd_amd import b1, synth
+
+
+def bf16_to_f32(bits: np.ndarray) -> np.ndarray:
+    return (bits.astype(np.uint32) << 16).view(np.float32)
+
+
+def parity(got: np.ndarray, ref: np.ndarray):
+    """(max-abs error / max|ref|, mean relative error) as the north star defines them."""
+    got = got.astype(np.float64)
+    ref = ref.astype(np.float64)
+    scale = np.max(np.abs(ref))
+    max_abs = np.max(np.abs(got - ref)) / scale
+    mean_rel = np.sum(np.abs(got - ref)) / np.sum(np.abs(ref))
+    return max_abs, mean_rel
+
+
+class DeviceLayer:
+    """Uploads canonical rank pools, prepares a layer, frees the canonical copies."""
+
+    def __init__(self, pools):
+        bufs = [b1.DeviceBuffer.from_host(p) for p in pools]
+        if len(bufs) == 1:
+            self.layer = b1.Layer(bufs[0].ptr, bufs[0].nbytes, 0)
+        else:
+            self.layer = b1.Layer.full([b.ptr for b in bufs], bufs[0].nbytes)
+        for b in bufs:
+            b.free()
+
+
+def run_ffn_dev(layer: b1.Layer, scratch: b1.Scratch, wl: synth.Workload, want_partial=True):
+    """Device-resident call; returns (stats, bf16 bits [rows,4096], fp32 partial or None)."""
+    dp = b1.DeviceBuffer.from_host(wl.payload)
+    ds = b1.DeviceBuffer.from_host(wl.scales)
+    di = b1.DeviceBuffer.from_host(wl.ids)
+    dw = b1.DeviceBuffer.from_host(wl.weights)
+    out = b1.DeviceBuffer(wl.rows * 4096 * 2)
+    part = b1.DeviceBuffer(wl.rows * 4096 * 4) if want_partial else None
+    stats = b1.ffn_dev(layer, scratch, dp.ptr, 4096, ds.ptr, 128, di.ptr, dw.ptr, wl.rows, out.ptr,
+                       part.ptr if part else None)
+    bf = out.to_host(np.uint16).reshape(wl.rows, 4096)
+    pf = part.to_host(np.float32).reshape(wl.rows, 4096) if part else None
+    return stats, bf, pf
