@@ -1,0 +1,232 @@
+"""GPU parity of the whole path through the C ABI against the CPU checker.
+
+Bars (the benchmark contract): bucketing and codec bytes bit-exact; outputs within
+max-abs <= 1e-2 * max|ref| and mean-rel <= 1e-3 of the CPU W4A8 reference, because the MFMA's FP32
+accumulation order differs from an FP64 dot. The requantised bytes are compared on the h the GPU
+reports, the reference's own rule (crates/mimo26-repack/tests/lattice_compare.py:105-108).
+"""
+import numpy as np
+import pytest
+
+import b1_oracle as O
+from helpers import DeviceLayer, bf16_to_f32, parity, run_ffn_dev
+from mimo26f_afd_amd import b1, synth
+from test_oracle_path import closed_form_image, closed_form_rows, exact_projection
+
+pytestmark = pytest.mark.gpu
+MAX_ABS, MEAN_REL = 1e-2, 1e-3
+# FP32 accumulation bound for one output: one rounding per 128-wide k-step plus the MFMA's internal
+# sum, against the FP64 ideal: a small multiple of 2^-24 times the sum of |products|.
+ACC_EPS = 8 * 2.0 ** -24
+
+
+def check_outputs(got_partial, got_bf16, ref_partial, ref_bf16):
+    ma, mr = parity(got_partial, ref_partial)
+    assert ma <= MAX_ABS and mr <= MEAN_REL, ("fp32 rank sum", ma, mr)
+    ma, mr = parity(bf16_to_f32(got_bf16), bf16_to_f32(ref_bf16))
+    assert ma <= MAX_ABS and mr <= MEAN_REL, ("bf16 rows", ma, mr)
+    return ma, mr
+
+
+def check_stages(scratch, layer, wl, pools, stats, experts=3):
+    """Plan bit-exact; per expert: gate/up/h within the accumulation bound, codec bytes exact on the
+    reported h, y within the output bars."""
+    n, inter = wl.rows * 8, layer.intermediate
+    ref = O.plan(max(256, wl.rows), wl.ids, wl.weights)
+    assert stats.groups == int(ref.group_count[0])
+    assert np.array_equal(scratch.view("original_routes", np.int32, n), ref.original_routes[:n])
+    assert np.array_equal(scratch.view("inverse", np.int32, n), ref.inverse[:n])
+    assert np.array_equal(scratch.view("grouped_weights", np.float32, n), ref.grouped_weights[:n])
+    groups = scratch.view("groups", O.GROUP_DTYPE, stats.groups)
+    assert np.array_equal(groups, ref.groups[:stats.groups])
+    rows_all = stats.groups * 16
+    taps = {k: scratch.view(k, np.float32, rows_all * inter).reshape(rows_all, inter) for k in ("gate", "up", "h")}
+    mp = scratch.view("mid_payload", np.uint8, rows_all * inter).reshape(rows_all, inter)
+    ms = scratch.view("mid_scales", np.uint8, rows_all * inter // 32).reshape(rows_all, inter // 32)
+    y = scratch.view("y", np.float32, n * 4096).reshape(n, 4096)
+    for gi in np.linspace(0, stats.groups - 1, experts).astype(int):
+        g = groups[gi]
+        r, toks = int(g["rows"]), g["input_rows"][:int(g["rows"])]
+        sl = slice(gi * 16, gi * 16 + r)
+        want = O.expert_ffn(pools, int(g["expert"]), wl.payload[toks], wl.scales[toks])
+        assert want["fault"] == 0
+        x = np.abs(O.activation_decode(wl.payload[toks], wl.scales[toks])[0].astype(np.float64))
+        for k in ("gate", "up"):
+            err = np.abs(taps[k][sl].astype(np.float64) - want[k])
+            assert np.max(err) <= ACC_EPS * 4096 * np.max(x) * 6 * 2.0 ** -4, (k, np.max(err))
+            assert parity(taps[k][sl], want[k])[1] < 1e-5
+        assert parity(taps["h"][sl], want["h"])[1] < 1e-4
+        assert np.array_equal(taps["h"][sl], O.silu_up(taps["gate"][sl], taps["up"][sl]))       # activation bit-exact on its inputs
+        qp, qs, qf = O.quant_v1(taps["h"][sl])
+        assert not qf.any() and np.array_equal(qp, mp[sl]) and np.array_equal(qs, ms[sl])       # codec bytes on the reported h
+        assert np.mean(mp[sl] == want["mid_payload"]) > 0.995
+        routes = ref.original_routes[int(g["route_base"]):int(g["route_base"]) + r]
+        ma, mr = parity(y[routes], want["y"])
+        assert ma <= MAX_ABS and mr <= MEAN_REL, ("y", ma, mr)
+
+
+@pytest.fixture(scope="module")
+def scratch():
+    s = b1.Scratch()
+    s.set_taps(True)
+    yield s
+    s.close()
+
+
+def test_closed_form_projections(scratch):
+    """The reference's synthetic projection fixture (tests/b1_core/compute_test.cuh:4-8,66-81) at the real
+    shapes N512/K4096 and N4096/K512, M in {1, 2, 4, 8, 16}, against exact sums; padded rows stay out."""
+    pool = np.full(synth.EXPERTS * synth.IMAGE_BYTES, 0x22, np.uint8)
+    imgs = {e: closed_form_image(e % 3) for e in (3, 77, 200)}
+    for e, img in imgs.items():
+        pool[e * synth.IMAGE_BYTES:(e + 1) * synth.IMAGE_BYTES] = img
+    layer = DeviceLayer([pool]).layer
+    assert layer.all_scales_normal() and layer.intermediate == 512
+    for m in (1, 2, 4, 8, 16):
+        payload, scales = closed_form_rows(m)
+        ids = np.tile(np.array([3, 77, 200, 1, 2, 4, 5, 6], np.int32), (m, 1))
+        w = np.tile(np.array([1, .5, .25, 0, 0, 0, 0, 0], np.float32), (m, 1))
+        wl = synth.Workload("closed form", -1, 0, 1, m, ids, w, np.zeros((m, 4096), np.float32), payload, scales)
+        stats, bf, pf = run_ffn_dev(layer, scratch, wl)
+        assert stats.groups == 8
+        groups = scratch.view("groups", O.GROUP_DTYPE, 8)
+        x64 = O.activation_decode(payload, scales)[0].astype(np.float64)
+        inter = 512
+        gate = scratch.view("gate", np.float32, 8 * 16 * inter).reshape(8 * 16, inter)
+        up = scratch.view("up", np.float32, 8 * 16 * inter).reshape(8 * 16, inter)
+        y = scratch.view("y", np.float32, m * 8 * 4096).reshape(m, 8, 4096)
+        mp = scratch.view("mid_payload", np.uint8, 8 * 16 * inter).reshape(8 * 16, inter)
+        ms = scratch.view("mid_scales", np.uint8, 8 * 16 * 16).reshape(8 * 16, 16)
+        for gi, g in enumerate(groups):
+            e = int(g["expert"])
+            if e not in imgs:
+                continue
+            assert int(g["rows"]) == m and g["input_rows"][:m].tolist() == list(range(m))
+            wg = exact_projection(imgs[e], 0, synth.GATE_SCALES, 512, 4096, x64)
+            wu = exact_projection(imgs[e], synth.UP_PAYLOAD, synth.UP_SCALES, 512, 4096, x64)
+            for got, want in ((gate[gi * 16:gi * 16 + m], wg), (up[gi * 16:gi * 16 + m], wu)):
+                assert np.all(np.abs(got.astype(np.float64) - want) <= 1e-5 + 1e-5 * np.abs(want) + ACC_EPS * np.max(np.abs(want)))
+            mid64 = O.activation_decode(mp[gi * 16:gi * 16 + m], ms[gi * 16:gi * 16 + m])[0].astype(np.float64)
+            wy = exact_projection(imgs[e], synth.DOWN_PAYLOAD, synth.DOWN_SCALES, 4096, 512, mid64)
+            slot = [3, 77, 200].index(e)
+            assert np.all(np.abs(y[:, slot].astype(np.float64) - wy) <= 1e-5 + 1e-5 * np.abs(wy) + ACC_EPS * np.max(np.abs(wy)))
+
+
+@pytest.mark.parametrize("cfg", [0, 1])
+def test_rank_share_configs(scratch, cfg):
+    """configs[0] (one expert: slot 0 carries weight 1) and configs[1] (256 experts, 16 tokens)."""
+    wl = synth.make(cfg)
+    pools = wl.pools(wl.touched())
+    layer = DeviceLayer(pools).layer
+    stats, bf, pf = run_ffn_dev(layer, scratch, wl)
+    rc, ref_partial, ref_bf16, ref_y = O.layer_ffn(pools, wl.payload, wl.scales, wl.ids, wl.weights, want_routes=True)
+    assert rc == 0
+    check_outputs(pf, bf, ref_partial, ref_bf16)
+    check_stages(scratch, layer, wl, pools, stats)
+    if cfg == 0:  # FP32 unweighted FC2 output of the single expert
+        y = scratch.view("y", np.float32, wl.rows * 8 * 4096).reshape(wl.rows, 8, 4096)[:, 0]
+        one = O.expert_ffn(pools, 0, wl.payload, wl.scales)["y"]
+        ma, mr = parity(y, one)
+        assert ma <= MAX_ABS and mr <= MEAN_REL
+    # the reference's host-pointer entry, separate arrays and in-frame rows of 4224 bytes
+    out = np.zeros((wl.rows, 4096), np.uint16)
+    st = b1.ffn(layer, scratch, wl.payload, wl.scales, wl.ids, wl.weights, wl.rows, out)
+    assert np.array_equal(out, bf) and st.groups == stats.groups and st.gpu_ms > 0
+    frame = np.zeros((wl.rows, 4224 + 64), np.uint8)
+    frame[:, :4096], frame[:, 4096:4224] = wl.payload, wl.scales
+    out2 = np.zeros((wl.rows, 4096), np.uint16)
+    b1.ffn_strided(layer, scratch, frame.reshape(-1), 4288, wl.ids, wl.weights, wl.rows, out2)
+    assert np.array_equal(out2, bf)
+
+
+@pytest.fixture(scope="module")
+def full_layer():
+    wl = synth.make(2)
+    pools = wl.pools()
+    return wl, pools, DeviceLayer(pools).layer
+
+
+def test_decode_layer_full_intermediate(scratch, full_layer):
+    """configs[2]: 256 experts x I 2048 on one GPU, 128 tokens, every row against the CPU reference."""
+    wl, pools, layer = full_layer
+    assert layer.intermediate == 2048
+    stats, bf, pf = run_ffn_dev(layer, scratch, wl)
+    rc, ref_partial, ref_bf16, _ = O.layer_ffn(pools, wl.payload, wl.scales, wl.ids, wl.weights)
+    assert rc == 0
+    check_outputs(pf, bf, ref_partial, ref_bf16)
+    check_stages(scratch, layer, wl, pools, stats)
+
+
+def test_prefill_chunk_properties_and_sampled_parity(full_layer):
+    """configs[3] at its full 8192 tokens: sampled rows against the CPU reference, and size-independent
+    properties over all rows: each row depends on its own routes only (a subset run alone reproduces
+    its rows bit for bit, a permuted batch permutes the rows), and the plan is a stable bijection."""
+    _, pools, layer = full_layer  # the same seeded weights serve both configurations
+    wl = synth.make(3)
+    s = b1.Scratch()
+    stats, bf, pf = run_ffn_dev(layer, s, wl)
+    n = wl.rows * 8
+    orig, inv = s.view("original_routes", np.int32, n), s.view("inverse", np.int32, n)
+    assert np.array_equal(np.sort(orig), np.arange(n)) and np.array_equal(inv[orig], np.arange(n))
+    experts = wl.ids.reshape(-1)[orig]
+    assert np.all(np.diff(experts) >= 0)
+    same = np.diff(experts) == 0
+    assert np.all(np.diff(orig)[same] > 0)                                 # stable inside every expert
+    sample = np.array([0, 1, 777, 4095, 4096, 8191])
+    sub = synth.Workload("sample", 3, wl.seed, 4, len(sample), wl.ids[sample], wl.weights[sample], wl.x[sample],
+                         wl.payload[sample], wl.scales[sample])
+    rc, ref_partial, ref_bf16, _ = O.layer_ffn(pools, sub.payload, sub.scales, sub.ids, sub.weights)
+    assert rc == 0
+    check_outputs(pf[sample], bf[sample], ref_partial, ref_bf16)
+    _, bf_sub, pf_sub = run_ffn_dev(layer, s, sub)
+    assert np.array_equal(bf_sub, bf[sample]) and np.array_equal(pf_sub.view(np.uint32), pf[sample].view(np.uint32))
+    perm = np.random.default_rng(1).permutation(wl.rows)
+    pw = synth.Workload("permuted", 3, wl.seed, 4, wl.rows, wl.ids[perm], wl.weights[perm], wl.x[perm], wl.payload[perm], wl.scales[perm])
+    _, bf_p, _ = run_ffn_dev(layer, s, pw, want_partial=False)
+    assert np.array_equal(bf_p, bf[perm])
+
+
+def test_errors_and_faults(full_layer):
+    """Return codes and messages of the reference entry (b1_serve.cu:315-317,365,551-562)."""
+    wl, pools, layer = full_layer
+    s = b1.Scratch()
+    out = np.zeros((wl.rows, 4096), np.uint16)
+    ids = wl.ids.copy(); ids[5, 3] = ids[5, 2]
+    with pytest.raises(b1.B1Error, match="invalid routes") as e:
+        b1.ffn(layer, s, wl.payload, wl.scales, ids, wl.weights, wl.rows, out)
+    assert e.value.code == 3
+    w = wl.weights.copy(); w[0, 0] = np.nan
+    with pytest.raises(b1.B1Error, match="invalid routes"):
+        b1.ffn(layer, s, wl.payload, wl.scales, wl.ids, w, wl.rows, out)
+    pay = wl.payload.copy(); pay[17, 100] = 0x7F                         # an E4M3 NaN code in one row
+    with pytest.raises(b1.B1Error, match="quantizer fault 1") as e:
+        b1.ffn(layer, s, pay, wl.scales, wl.ids, wl.weights, wl.rows, out)
+    assert e.value.code == 4 and O.layer_ffn(pools, pay[16:18], wl.scales[16:18], wl.ids[16:18], wl.weights[16:18])[0] == 4
+    sc = wl.scales.copy(); sc[3, 9] = 104                                # activation scale below the legal window
+    with pytest.raises(b1.B1Error, match="quantizer fault 1"):
+        b1.ffn(layer, s, wl.payload, sc, wl.ids, wl.weights, wl.rows, out)
+    from mimo26f_afd_amd._lib import load
+    import ctypes as C
+    buf = C.create_string_buffer(256)
+    lib = load()
+    args = (wl.payload.ctypes.data, 4096, wl.scales.ctypes.data, 128, wl.ids.ctypes.data, wl.weights.ctypes.data)
+    assert lib.m26s_b1_ffn(layer._h, s._h, *args, 0, out.ctypes.data, None, buf, 256) == 1
+    assert lib.m26s_b1_ffn(layer._h, s._h, *args, 8193, out.ctypes.data, None, buf, 256) == 1
+    assert lib.m26s_b1_ffn(layer._h, s._h, args[0], 4095, *args[2:], 16, out.ctypes.data, None, buf, 256) == 1
+    assert lib.m26s_b1_ffn(None, s._h, *args, 16, out.ctypes.data, None, buf, 256) == 1 and b"bad rows/handles/pitch" in buf.value
+    assert lib.m26s_b1_layer_new(1, 5, 0, C.byref(C.c_void_p()), buf, 256) == 1 and b"bad canonical extent/rank" in buf.value
+    st = b1.ffn(layer, s, wl.payload, wl.scales, wl.ids, wl.weights, wl.rows, out)   # the scratch recovers after faults
+    assert st.groups > 0 and out.any()
+
+
+def test_abnormal_weight_scales_are_refused():
+    """A weight scale byte outside [2,252] clears all_normal (b1_fc1_m64.cuh:496-512); the MFMA path is
+    then refused loudly instead of computing with a NaN or saturating scale."""
+    wl = synth.make(1)
+    pools = wl.pools(wl.touched())
+    pools[0][int(wl.ids[0, 0]) * synth.IMAGE_BYTES + synth.GATE_SCALES + 5] = 255
+    layer = DeviceLayer(pools).layer
+    assert not layer.all_scales_normal()
+    with pytest.raises(b1.B1Error, match="outside") as e:
+        b1.ffn(layer, b1.Scratch(), wl.payload, wl.scales, wl.ids, wl.weights, wl.rows, np.zeros((wl.rows, 4096), np.uint16))
+    assert e.value.code == 4
