@@ -342,71 +342,74 @@ __global__ void __launch_bounds__(256) quantize_kernel(const float* __restrict__
 // Block-scaled grouped GEMM core, shared by FC1 and FC2.
 //
 // One wave owns four 16-row weight tiles (SrcA, FP4, streamed once, fully coalesced 1 KB per
-// tile per k-step) and up to NT 16-row activation tiles (SrcB, FP8, row-major rows gathered by
+// tile per k-step) and TT 16-row activation tiles (SrcB, FP8, row-major rows gathered by
 // pointer). A k-step is K = 128. Loads for step k+1 are issued before the MFMAs of step k.
+// The walk over K starts at quad `first` and wraps, so waves that stream neighbouring weight
+// blocks do not sit on the same addresses modulo the block size at the same time.
 // ---------------------------------------------------------------------------------------------
-template <int NT>
+template <int TT>
 struct Operands {
     v4i a[4];
-    v4i lo[NT], hi[NT];
-    uint32_t sb[NT];
+    v4i lo[TT], hi[TT];
+    uint32_t sb[TT];
 };
 
-template <int NT>
-__device__ __forceinline__ void load_step(Operands<NT>& o, const uint8_t* __restrict__ wp, int ks,
-                                          const uint8_t* const (&xrow)[NT], const uint8_t* const (&xsrow)[NT],
-                                          int tiles) {
+template <int TT>
+__device__ __forceinline__ void load_step(Operands<TT>& o, const uint8_t* __restrict__ wp, int ks,
+                                          const uint8_t* const (&xrow)[TT], const uint8_t* const (&xsrow)[TT]) {
 #pragma unroll
-    for (int t = 0; t < 4; ++t) o.a[t] = *reinterpret_cast<const v4i*>(wp + size_t(ks) * 4096 + t * 1024);
+    for (int t = 0; t < 4; ++t) o.a[t] = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(wp + size_t(ks) * 4096 + t * 1024));
 #pragma unroll
-    for (int tt = 0; tt < NT; ++tt)
-        if (tt < tiles) {
-            o.lo[tt] = *reinterpret_cast<const v4i*>(xrow[tt] + ks * 128);
-            o.hi[tt] = *reinterpret_cast<const v4i*>(xrow[tt] + ks * 128 + 64);
-            o.sb[tt] = *reinterpret_cast<const uint32_t*>(xsrow[tt] + ks * 4);
-        }
+    for (int tt = 0; tt < TT; ++tt) {
+        o.lo[tt] = *reinterpret_cast<const v4i*>(xrow[tt] + ks * 128);
+        o.hi[tt] = *reinterpret_cast<const v4i*>(xrow[tt] + ks * 128 + 64);
+        o.sb[tt] = *reinterpret_cast<const uint32_t*>(xsrow[tt] + ks * 4);
+    }
 }
 
-template <int NT, int SEL>
-__device__ __forceinline__ void mfma_step(v4f (&acc)[4][NT], const Operands<NT>& o, const uint32_t (&sw)[4],
-                                          int tiles, uint32_t shift, uint32_t& bad) {
+template <int TT, int SEL>
+__device__ __forceinline__ void mfma_step(v4f (&acc)[4][TT], const Operands<TT>& o, const uint32_t (&sw)[4],
+                                          uint32_t shift, uint32_t& bad) {
 #pragma unroll
-    for (int tt = 0; tt < NT; ++tt)
-        if (tt < tiles) {
-            const uint32_t s = (o.sb[tt] >> shift) & 0xffu;
-            bad |= (s - 105u) > 142u ? 1u : 0u;  // activation scales are legal only in [105, 247]
-            const v8i b = {o.lo[tt].x, o.lo[tt].y, o.lo[tt].z, o.lo[tt].w, o.hi[tt].x, o.hi[tt].y, o.hi[tt].z, o.hi[tt].w};
+    for (int tt = 0; tt < TT; ++tt) {
+        const uint32_t s = (o.sb[tt] >> shift) & 0xffu;
+        bad |= (s - 105u) > 142u ? 1u : 0u;  // activation scales are legal only in [105, 247]
+        const v8i b = {o.lo[tt].x, o.lo[tt].y, o.lo[tt].z, o.lo[tt].w, o.hi[tt].x, o.hi[tt].y, o.hi[tt].z, o.hi[tt].w};
 #pragma unroll
-            for (int t = 0; t < 4; ++t) {
-                const v8i a = {o.a[t].x, o.a[t].y, o.a[t].z, o.a[t].w, 0, 0, 0, 0};
-                acc[t][tt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, acc[t][tt], 4 /*A: E2M1*/,
-                                                                              0 /*B: E4M3*/, SEL, int(sw[t]), 0, int(s));
-            }
+        for (int t = 0; t < 4; ++t) {
+            const v8i a = {o.a[t].x, o.a[t].y, o.a[t].z, o.a[t].w, 0, 0, 0, 0};
+            acc[t][tt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, acc[t][tt], 4 /*A: E2M1*/,
+                                                                          0 /*B: E4M3*/, SEL, int(sw[t]), 0, int(s));
         }
+    }
 }
 
 // wp / sp already include the lane offset (lane*16, lane*4). ksteps is a multiple of 4.
-template <int NT>
-__device__ __forceinline__ void gemm_chunk(v4f (&acc)[4][NT], const uint8_t* __restrict__ wp,
-                                           const uint8_t* __restrict__ sp, int ksteps,
-                                           const uint8_t* const (&xrow)[NT], const uint8_t* const (&xsrow)[NT],
-                                           int tiles, uint32_t lane, uint32_t& bad) {
+template <int TT>
+__device__ __forceinline__ void gemm_chunk(v4f (&acc)[4][TT], const uint8_t* __restrict__ wp,
+                                           const uint8_t* __restrict__ sp, int ksteps, int first,
+                                           const uint8_t* const (&xrow)[TT], const uint8_t* const (&xsrow)[TT],
+                                           uint32_t lane, uint32_t& bad) {
     const uint32_t shift = 8 * (lane >> 4);
-    Operands<NT> cur, nxt;
-    load_step<NT>(cur, wp, 0, xrow, xsrow, tiles);
-    for (int q = 0; q < ksteps / 4; ++q) {
+    const int quads = ksteps / 4;
+    Operands<TT> cur, nxt;
+    int q = first;
+    load_step<TT>(cur, wp, 4 * q, xrow, xsrow);
+    for (int i = 0; i < quads; ++i) {
         uint32_t sw[4];
 #pragma unroll
         for (int t = 0; t < 4; ++t) sw[t] = *reinterpret_cast<const uint32_t*>(sp + size_t(q) * 1024 + t * 256);
         const int ks = 4 * q;
-        load_step<NT>(nxt, wp, ks + 1, xrow, xsrow, tiles);
-        mfma_step<NT, 0>(acc, cur, sw, tiles, shift, bad);
-        load_step<NT>(cur, wp, ks + 2, xrow, xsrow, tiles);
-        mfma_step<NT, 1>(acc, nxt, sw, tiles, shift, bad);
-        load_step<NT>(nxt, wp, ks + 3, xrow, xsrow, tiles);
-        mfma_step<NT, 2>(acc, cur, sw, tiles, shift, bad);
-        if (ks + 4 < ksteps) load_step<NT>(cur, wp, ks + 4, xrow, xsrow, tiles);
-        mfma_step<NT, 3>(acc, nxt, sw, tiles, shift, bad);
+        const int qn = q + 1 == quads ? 0 : q + 1;
+        load_step<TT>(nxt, wp, ks + 1, xrow, xsrow);
+        mfma_step<TT, 0>(acc, cur, sw, shift, bad);
+        load_step<TT>(cur, wp, ks + 2, xrow, xsrow);
+        mfma_step<TT, 1>(acc, nxt, sw, shift, bad);
+        load_step<TT>(nxt, wp, ks + 3, xrow, xsrow);
+        mfma_step<TT, 2>(acc, cur, sw, shift, bad);
+        if (i + 1 < quads) load_step<TT>(cur, wp, 4 * qn, xrow, xsrow);
+        mfma_step<TT, 3>(acc, nxt, sw, shift, bad);
+        q = qn;
     }
 }
 
@@ -437,30 +440,19 @@ struct Fc1Args {
     float* tap_h;
 };
 
-// Stages 2+3: gate/up grouped GEMM, SwiGLU and the v1 requantisation of the intermediate.
-// grid (I/128, chunk capacity), 256 threads; each wave owns one 32-column K32 block of the
-// intermediate for every row of its chunk, so a quantizer block never leaves the wave.
-template <int NT>
-__global__ void __launch_bounds__(256) fc1_kernel(Fc1Args a) {
+// One wave's share of FC1 for a chunk of TT groups: 32 intermediate columns x 16*TT rows.
+template <int TT>
+__device__ __forceinline__ void fc1_body(const Fc1Args& a, const Chunk ch, uint32_t cb, uint32_t lane) {
     uint32_t* meta = a.plan.meta;
-    const uint32_t c = blockIdx.y;
-    if (meta[kPlanFault] || c >= meta[kChunkCount]) return;
-    const Chunk ch = a.plan.chunks[c];
-    const uint32_t lane = threadIdx.x & 63, wv = threadIdx.x >> 6, r = lane & 15, g = lane >> 4;
-    const uint32_t I = a.lay.inter, cb = blockIdx.x * 4 + wv;
-    const int tiles = ch.groups < NT ? ch.groups : NT;
+    const uint32_t r = lane & 15, g = lane >> 4, I = a.lay.inter;
     const Group* grp = a.plan.groups + ch.first_group;
     const int32_t expert = grp[0].expert;
-    if (expert < 0 || expert >= int32_t(kExperts) || tiles < 1) {
-        if (lane == 0) atomicOr(&meta[kFc1Fault], 2u);
-        return;
-    }
-    const uint8_t* xrow[NT];
-    const uint8_t* xsrow[NT];
-    bool live[NT];
+    const uint8_t* xrow[TT];
+    const uint8_t* xsrow[TT];
+    bool live[TT];
 #pragma unroll
-    for (int tt = 0; tt < NT; ++tt) {
-        const int32_t row = tt < tiles ? grp[tt].input_rows[r] : -1;
+    for (int tt = 0; tt < TT; ++tt) {
+        const int32_t row = tt < ch.groups ? grp[tt].input_rows[r] : -1;
         live[tt] = row >= 0;
         xrow[tt] = (live[tt] ? a.x + size_t(row) * a.x_pitch : a.zero_row) + g * 16;
         xsrow[tt] = live[tt] ? a.xs + size_t(row) * a.xs_pitch : a.unit_scales;
@@ -468,19 +460,18 @@ __global__ void __launch_bounds__(256) fc1_kernel(Fc1Args a) {
     const uint8_t* img = a.prepared + uint64_t(expert) * a.lay.bytes();
     const uint8_t* wp = img + a.lay.w13() + uint64_t(cb) * (32 * 4096) + lane * 16;
     const uint8_t* sp = img + a.lay.s13() + uint64_t(cb) * (8 * 1024) + lane * 4;
-    v4f acc[4][NT];
+    v4f acc[4][TT];
 #pragma unroll
     for (int t = 0; t < 4; ++t)
 #pragma unroll
-        for (int tt = 0; tt < NT; ++tt) acc[t][tt] = v4f{0.f, 0.f, 0.f, 0.f};
+        for (int tt = 0; tt < TT; ++tt) acc[t][tt] = v4f{0.f, 0.f, 0.f, 0.f};
     uint32_t bad = 0;
-    gemm_chunk<NT>(acc, wp, sp, 32, xrow, xsrow, tiles, lane, bad);
+    gemm_chunk<TT>(acc, wp, sp, 32, int(cb & 7), xrow, xsrow, lane, bad);
     bad |= __shfl_xor(bad, 16);
     bad |= __shfl_xor(bad, 32);
 
 #pragma unroll
-    for (int tt = 0; tt < NT; ++tt) {
-        if (tt >= tiles) continue;
+    for (int tt = 0; tt < TT; ++tt) {
         float h[2][4];
         uint32_t amax = 0;
 #pragma unroll
@@ -509,20 +500,18 @@ __global__ void __launch_bounds__(256) fc1_kernel(Fc1Args a) {
         uint32_t fault = (amax >= 0x7f800000u || bad) ? 1u : 0u;
         const int k = quant_scale_exponent(amax);
         uint32_t word[2] = {0, 0};
-        if (!fault) {
-            uint32_t over = 0;
+        uint32_t over = 0;
 #pragma unroll
-            for (int t2 = 0; t2 < 2; ++t2)
+        for (int t2 = 0; t2 < 2; ++t2)
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const uint32_t code = quant_code(__float_as_uint(h[t2][i]), k);
-                    over |= quant_reconstructs(code, k) ? 0u : 1u;
-                    word[t2] |= code << (8 * i);
-                }
-            over |= __shfl_xor(over, 16);
-            over |= __shfl_xor(over, 32);
-            if (over) fault = 2;
-        }
+            for (int i = 0; i < 4; ++i) {
+                const uint32_t code = quant_code(__float_as_uint(h[t2][i]), k);
+                over |= quant_reconstructs(code, k) ? 0u : 1u;
+                word[t2] |= code << (8 * i);
+            }
+        over |= __shfl_xor(over, 16);
+        over |= __shfl_xor(over, 32);
+        if (!fault && over) fault = 2;
         if (!live[tt]) continue;
         if (fault) {
             if (g == 0) {
@@ -537,6 +526,28 @@ __global__ void __launch_bounds__(256) fc1_kernel(Fc1Args a) {
     }
 }
 
+// Stages 2+3: gate/up grouped GEMM, SwiGLU and the v1 requantisation of the intermediate.
+// grid (I/128, chunk capacity), 256 threads; each wave owns one 32-column K32 block of the
+// intermediate for every row of its chunk, so a quantizer block never leaves the wave. A chunk
+// holds at most NT groups; the body is compiled for 1, 2, 4 and 8 activation tiles.
+template <int NT>
+__global__ void __launch_bounds__(256) fc1_kernel(Fc1Args a) {
+    uint32_t* meta = a.plan.meta;
+    const uint32_t c = blockIdx.y;
+    if (meta[kPlanFault] || c >= meta[kChunkCount]) return;
+    const Chunk ch = a.plan.chunks[c];
+    const uint32_t lane = threadIdx.x & 63, cb = blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int32_t expert = a.plan.groups[ch.first_group].expert;
+    if (expert < 0 || expert >= int32_t(kExperts) || ch.groups < 1 || ch.groups > NT) {
+        if (lane == 0) atomicOr(&meta[kFc1Fault], 2u);
+        return;
+    }
+    if (NT == 1 || ch.groups == 1) fc1_body<1>(a, ch, cb, lane);
+    else if (NT == 2 || ch.groups == 2) fc1_body<2>(a, ch, cb, lane);
+    else if (NT >= 4 && ch.groups <= 4) fc1_body<(NT >= 4 ? 4 : 1)>(a, ch, cb, lane);
+    else fc1_body<(NT >= 8 ? 8 : 1)>(a, ch, cb, lane);
+}
+
 struct Fc2Args {
     const uint8_t* prepared;
     Prepared lay;
@@ -549,29 +560,18 @@ struct Fc2Args {
     uint32_t routes;
 };
 
-// Stage 4a: down grouped GEMM on the requantised intermediate; rows go back to y[original route].
-// grid (16, chunk capacity), 256 threads; each wave owns 64 output columns.
-template <int NT>
-__global__ void __launch_bounds__(256) fc2_kernel(Fc2Args a) {
-    uint32_t* meta = a.plan.meta;
-    const uint32_t c = blockIdx.y;
-    if (meta[kPlanFault] || meta[kFc1Fault] || meta[kQuantFault] || c >= meta[kChunkCount]) return;
-    const Chunk ch = a.plan.chunks[c];
-    const uint32_t lane = threadIdx.x & 63, wv = threadIdx.x >> 6, r = lane & 15, g = lane >> 4;
-    const uint32_t I = a.lay.inter, ob = blockIdx.x * 4 + wv;
-    const int tiles = ch.groups < NT ? ch.groups : NT;
+// One wave's share of FC2 for a chunk of TT groups: 64 output columns x 16*TT rows.
+template <int TT>
+__device__ __forceinline__ void fc2_body(const Fc2Args& a, const Chunk ch, uint32_t ob, uint32_t lane) {
+    const uint32_t r = lane & 15, g = lane >> 4, I = a.lay.inter;
     const Group* grp = a.plan.groups + ch.first_group;
     const int32_t expert = grp[0].expert;
-    if (expert < 0 || expert >= int32_t(kExperts) || tiles < 1) {
-        if (lane == 0) atomicOr(&meta[kFc2Fault], 2u);
-        return;
-    }
-    const uint8_t* xrow[NT];
-    const uint8_t* xsrow[NT];
-    int32_t route[NT];
+    const uint8_t* xrow[TT];
+    const uint8_t* xsrow[TT];
+    int32_t route[TT];
 #pragma unroll
-    for (int tt = 0; tt < NT; ++tt) {
-        const bool live = tt < tiles && int32_t(r) < grp[tt].rows;
+    for (int tt = 0; tt < TT; ++tt) {
+        const bool live = tt < ch.groups && int32_t(r) < grp[tt].rows;
         const size_t grow = size_t(ch.first_group + tt) * 16 + r;
         route[tt] = live ? a.plan.original[grp[tt].route_base + r] : -1;
         xrow[tt] = (live ? a.dq + grow * I : a.zero_row) + g * 16;
@@ -581,23 +581,43 @@ __global__ void __launch_bounds__(256) fc2_kernel(Fc2Args a) {
     const uint8_t* img = a.prepared + uint64_t(expert) * a.lay.bytes();
     const uint8_t* wp = img + a.lay.w2() + uint64_t(ob) * ksteps * 4096 + lane * 16;
     const uint8_t* sp = img + a.lay.s2() + uint64_t(ob) * (ksteps / 4) * 1024 + lane * 4;
-    v4f acc[4][NT];
+    v4f acc[4][TT];
 #pragma unroll
     for (int t = 0; t < 4; ++t)
 #pragma unroll
-        for (int tt = 0; tt < NT; ++tt) acc[t][tt] = v4f{0.f, 0.f, 0.f, 0.f};
+        for (int tt = 0; tt < TT; ++tt) acc[t][tt] = v4f{0.f, 0.f, 0.f, 0.f};
     uint32_t bad = 0;
-    gemm_chunk<NT>(acc, wp, sp, int(ksteps), xrow, xsrow, tiles, lane, bad);
+    gemm_chunk<TT>(acc, wp, sp, int(ksteps), int(ob % (ksteps / 4)), xrow, xsrow, lane, bad);
     bool lost = false;
 #pragma unroll
-    for (int tt = 0; tt < NT; ++tt) {
-        if (tt >= tiles || route[tt] < 0) continue;
+    for (int tt = 0; tt < TT; ++tt) {
+        if (route[tt] < 0) continue;
         if (uint32_t(route[tt]) >= a.routes) { lost = true; continue; }
         float* dst = a.y + size_t(route[tt]) * kHidden + ob * 64 + 4 * g;
 #pragma unroll
         for (int t = 0; t < 4; ++t) *reinterpret_cast<v4f*>(dst + 16 * t) = acc[t][tt];
     }
-    if (lost) atomicOr(&meta[kFc2Fault], 5u);
+    if (lost) atomicOr(&a.plan.meta[kFc2Fault], 5u);
+}
+
+// Stage 4a: down grouped GEMM on the requantised intermediate; rows go back to y[original route].
+// grid (16, chunk capacity), 256 threads; each wave owns 64 output columns.
+template <int NT>
+__global__ void __launch_bounds__(256) fc2_kernel(Fc2Args a) {
+    uint32_t* meta = a.plan.meta;
+    const uint32_t c = blockIdx.y;
+    if (meta[kPlanFault] || meta[kFc1Fault] || meta[kQuantFault] || c >= meta[kChunkCount]) return;
+    const Chunk ch = a.plan.chunks[c];
+    const uint32_t lane = threadIdx.x & 63, ob = blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int32_t expert = a.plan.groups[ch.first_group].expert;
+    if (expert < 0 || expert >= int32_t(kExperts) || ch.groups < 1 || ch.groups > NT) {
+        if (lane == 0) atomicOr(&meta[kFc2Fault], 2u);
+        return;
+    }
+    if (NT == 1 || ch.groups == 1) fc2_body<1>(a, ch, ob, lane);
+    else if (NT == 2 || ch.groups == 2) fc2_body<2>(a, ch, ob, lane);
+    else if (NT >= 4 && ch.groups <= 4) fc2_body<(NT >= 4 ? 4 : 1)>(a, ch, ob, lane);
+    else fc2_body<(NT >= 8 ? 8 : 1)>(a, ch, ob, lane);
 }
 
 // Stage 4b: router-weighted combine. Per (token, column): v = 0; for slot 0..7:
