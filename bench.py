@@ -85,12 +85,14 @@ def kernel_phases(layer, scratch, d, rows, reps, b1):
 
 
 def sample_parity(wl, pools, got_bits, tokens, O):
-    """GPU BF16 rows against the CPU checker on a few tokens."""
-    ref_rc, ref_partial, _, _ = O.layer_ffn(pools, wl.payload[tokens], wl.scales[tokens], wl.ids[tokens], wl.weights[tokens])
+    """GPU BF16 rows against the CPU checker's BF16 rows on a few tokens (like with like: both sides
+    carry the one BF16 rounding of the rank sum)."""
+    ref_rc, _, ref_bits, _ = O.layer_ffn(pools, wl.payload[tokens], wl.scales[tokens], wl.ids[tokens], wl.weights[tokens])
     got = (got_bits[tokens].astype(np.uint32) << 16).view(np.float32).astype(np.float64)
-    ref = ref_partial.astype(np.float64)
+    ref = (ref_bits.astype(np.uint32) << 16).view(np.float32).astype(np.float64)
     return dict(tokens=len(tokens), oracle_rc=ref_rc, max_abs_over_max_ref=float(np.max(np.abs(got - ref)) / np.max(np.abs(ref))),
-                mean_rel=float(np.sum(np.abs(got - ref)) / np.sum(np.abs(ref))))
+                mean_rel=float(np.sum(np.abs(got - ref)) / np.sum(np.abs(ref))),
+                bf16_identical_fraction=float(np.mean(got_bits[tokens] == ref_bits)))
 
 
 def cpu_baseline(wl, pools, tokens, O):
