@@ -134,6 +134,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-prefill", action="store_true", help="skip the 8192-token prefill measurement")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--only-prefill", action="store_true",
+                    help="profiling aid: run only the prefill measurement and print its object")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU only (no collectives, no sharding); use --gpus 1")
@@ -146,6 +148,10 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
 
+    if args.only_prefill:
+        pre = run_config(3, args.steps, args.warmup, torch, dev, b1, synth, O, parity_tokens=2, cpu_tokens=0)
+        print(json.dumps(dict(ms_per_step=pre["ms_per_step"], phases=pre["phases"], parity=pre["parity"])), flush=True)
+        return
     dec = run_config(2, args.steps, args.warmup, torch, dev, b1, synth, O, parity_tokens=8,
                      cpu_tokens=0 if args.no_cpu else 128)
     wl = dec["wl"]

@@ -41,9 +41,10 @@ def load() -> C.CDLL:
     """The built library; built first only if nothing is there."""
     global _LIB
     if _LIB is None:
-        if not os.path.exists(build.LIB):
+        path = os.environ.get("M26S_B1_LIB") or build.LIB  # a deployment may point at its own build
+        if path == build.LIB and not os.path.exists(path):
             build.build_library()
-        lib = C.CDLL(build.LIB)
+        lib = C.CDLL(path)
         for name, (res, args) in SIGNATURES.items():
             fn = getattr(lib, name)  # AttributeError here = a declared symbol is not exported
             fn.restype = res

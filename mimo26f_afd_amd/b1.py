@@ -75,7 +75,7 @@ class Layer:
         return int(load().m26s_b1_layer_intermediate(self._h))
 
     def close(self) -> None:
-        if getattr(self, "_h", None) and self._h.value:
+        if getattr(self, "_h", None) and self._h.value and load is not None:  # load is gone at interpreter exit
             load().m26s_b1_layer_free(self._h)
             self._h = C.c_void_p()
 
@@ -116,7 +116,7 @@ class Scratch:
         return out
 
     def close(self) -> None:
-        if getattr(self, "_h", None) and self._h.value:
+        if getattr(self, "_h", None) and self._h.value and load is not None:
             load().m26s_b1_scratch_free(self._h)
             self._h = C.c_void_p()
 
@@ -225,7 +225,7 @@ class DeviceBuffer:
         return out
 
     def free(self) -> None:
-        if getattr(self, "ptr", None):
+        if getattr(self, "ptr", None) and load is not None:
             load().m26s_b1_device_free(self.ptr)
             self.ptr = None
 

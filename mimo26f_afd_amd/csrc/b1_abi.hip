@@ -11,7 +11,7 @@
 #include <vector>
 
 #include "../../include/m26s_b1.h"
-#include "b1_kernels.h"
+#include "b1_tile.h"
 
 using namespace m26g;
 
@@ -52,12 +52,19 @@ uint64_t chunk_bound(uint64_t routes, uint32_t gpc) {
 // weights for up to 32 rows; larger calls reuse each weight fragment over 128 rows.
 uint32_t tiles_for(uint32_t rows) { return rows <= 32 ? 1u : rows <= 512 ? 2u : 8u; }
 
-bool plan_lds_ready = false;
+// Kernels whose dynamic LDS passes 64 KB need the limit raised once per process.
+bool lds_ready = false;
 hipError_t plan_lds_attr() {
-    if (plan_lds_ready) return hipSuccess;
-    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(plan_kernel),
-                                             hipFuncAttributeMaxDynamicSharedMemorySize, int(kMaxRows * kTopk));
-    plan_lds_ready = e == hipSuccess;
+    if (lds_ready) return hipSuccess;
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(plan_kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, int(kMaxRows * kTopk));
+    if (e == hipSuccess)
+        e = hipFuncSetAttribute(reinterpret_cast<const void*>(fc1_tile_kernel),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, int(tile_lds_bytes(8, kHidden)));
+    if (e == hipSuccess)
+        e = hipFuncSetAttribute(reinterpret_cast<const void*>(fc2_tile_kernel),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, int(tile_lds_bytes(8, 4 * kRankI)));
+    lds_ready = e == hipSuccess;
     return e;
 }
 
@@ -158,6 +165,22 @@ void launch_ffn(const m26s_b1_layer* L, m26s_b1_scratch* S, const PlanView& pv, 
     (void)hipEventRecord(S->ec, S->st);
 }
 
+// Prefill-size calls: 512-thread workgroups that share each chunk's activation tiles through LDS.
+void launch_tiles(const m26s_b1_layer* L, m26s_b1_scratch* S, const PlanView& pv, const uint8_t* x, size_t xp,
+                  const uint8_t* xs, size_t xsp, uint32_t chunk_cap, uint64_t routes) {
+    const uint8_t* zero = S->pad.as<uint8_t>();
+    const uint32_t inter = L->lay.inter;
+    Fc1Args f1{L->prepared, L->lay, pv, x, xp, xs, xsp, zero, zero + 8192, S->dq.as<uint8_t>(), S->dqs.as<uint8_t>(),
+               S->taps ? S->tap_gate.as<float>() : nullptr, S->taps ? S->tap_up.as<float>() : nullptr,
+               S->taps ? S->tap_h.as<float>() : nullptr};
+    fc1_tile_kernel<<<dim3(inter / 256, chunk_cap), kTileThreads, tile_lds_bytes(8, kHidden), S->st>>>(f1);
+    (void)hipEventRecord(S->ea, S->st);
+    Fc2Args f2{L->prepared, L->lay, pv, S->dq.as<uint8_t>(), S->dqs.as<uint8_t>(), zero, zero + 8192,
+               S->y.as<float>(), uint32_t(routes)};
+    fc2_tile_kernel<<<dim3(8, chunk_cap), kTileThreads, tile_lds_bytes(8, inter), S->st>>>(f2);
+    (void)hipEventRecord(S->ec, S->st);
+}
+
 // Enqueue plan -> FC1(+quantizer) -> FC2 -> reduce on device-resident inputs. No host wait.
 int enqueue(const m26s_b1_layer* L, m26s_b1_scratch* S, const uint8_t* x, size_t xp, const uint8_t* xs, size_t xsp,
             const int32_t* ids, const float* w, uint32_t rows, uint16_t* bf16_out, float* partial, char* err,
@@ -188,7 +211,7 @@ int enqueue(const m26s_b1_layer* L, m26s_b1_scratch* S, const uint8_t* x, size_t
     M26S_CK(hipEventRecord(S->ep, S->st), "b1 event p");
     if (nt == 1) launch_ffn<1>(L, S, pv, x, xp, xs, xsp, uint32_t(ccap), routes);
     else if (nt == 2) launch_ffn<2>(L, S, pv, x, xp, xs, xsp, uint32_t(ccap), routes);
-    else launch_ffn<8>(L, S, pv, x, xp, xs, xsp, uint32_t(ccap), routes);
+    else launch_tiles(L, S, pv, x, xp, xs, xsp, uint32_t(ccap), routes);
     M26S_CK(hipGetLastError(), "b1 fc launch");
     const uint64_t n4 = uint64_t(rows) * (kHidden / 4);
     const uint32_t blocks = uint32_t(n4 / 256 < 8192 ? (n4 + 255) / 256 : 8192);

@@ -413,11 +413,36 @@ __device__ __forceinline__ void gemm_chunk(v4f (&acc)[4][TT], const uint8_t* __r
     }
 }
 
-// SwiGLU in the reference's stable form (kernels/b1/grouped.cu:89-93) with the CPU reference's
-// exponential: binary64 exp rounded once to binary32 (mimo26-repack/tests/lattice_oracle.py:32-53).
+// e^t for t <= 0 as the CPU reference forms it: evaluated in binary64, rounded once to binary32
+// (mimo26-repack/tests/lattice_oracle.py:32-53 uses libm's binary64 exp). Cody-Waite reduction by
+// ln 2 and an 11th-degree Taylor polynomial on |r| <= 0.347 keep the binary64 value within a few
+// ulp (2^-47 truncation), so the binary32 rounding differs from libm's only when the exact value
+// lies within ~1e-15 of a rounding boundary. About twenty FP64 operations, few live registers.
+__device__ __forceinline__ float exp_nonpositive(float tf) {
+    const double t = double(tf);
+    const double n = __builtin_rint(t * 1.4426950408889634074);
+    double r = __builtin_fma(n, -6.93147180369123816490e-01, t);
+    r = __builtin_fma(n, -1.90821492927058770002e-10, r);
+    double p = 2.50521083854417187751e-08;  // 1/11!
+    p = __builtin_fma(p, r, 2.75573192239858906526e-07);
+    p = __builtin_fma(p, r, 2.75573192239858906526e-06);
+    p = __builtin_fma(p, r, 2.48015873015873015873e-05);
+    p = __builtin_fma(p, r, 1.98412698412698412698e-04);
+    p = __builtin_fma(p, r, 1.38888888888888888889e-03);
+    p = __builtin_fma(p, r, 8.33333333333333333333e-03);
+    p = __builtin_fma(p, r, 4.16666666666666666667e-02);
+    p = __builtin_fma(p, r, 1.66666666666666666667e-01);
+    p = __builtin_fma(p, r, 0.5);
+    p = __builtin_fma(p, r, 1.0);
+    p = __builtin_fma(p, r, 1.0);
+    return float(__builtin_ldexp(p, int(n)));
+}
+
+// SwiGLU in the reference's stable form (kernels/b1/grouped.cu:89-93): e = exp(-|g|);
+// s = g >= 0 ? g/(1+e) : (g*e)/(1+e); h = s*u, every step one FP32 rounding.
 __device__ __forceinline__ float silu_up(float g, float u) {
     const float t = g >= 0.0f ? -g : g;
-    const float e = float(exp(double(t)));
+    const float e = exp_nonpositive(t);
     const float d = __fadd_rn(1.0f, e);
     const float s = g >= 0.0f ? __fdiv_rn(g, d) : __fdiv_rn(__fmul_rn(g, e), d);
     return __fmul_rn(s, u);
@@ -440,33 +465,14 @@ struct Fc1Args {
     float* tap_h;
 };
 
-// One wave's share of FC1 for a chunk of TT groups: 32 intermediate columns x 16*TT rows.
+// FC1 epilogue of one wave: SwiGLU on the gate/up accumulators, then quantizer v1 of each row's
+// 32-column block straight from registers (amax across the four lanes that share a row, frexp-rule
+// exponent, exact-grid RNE, reconstruction check), packed stores of payload and scale.
 template <int TT>
-__device__ __forceinline__ void fc1_body(const Fc1Args& a, const Chunk ch, uint32_t cb, uint32_t lane) {
+__device__ __forceinline__ void fc1_finish(const Fc1Args& a, const Chunk ch, uint32_t cb, uint32_t lane,
+                                           v4f (&acc)[4][TT], uint32_t bad, const bool (&live)[TT]) {
     uint32_t* meta = a.plan.meta;
     const uint32_t r = lane & 15, g = lane >> 4, I = a.lay.inter;
-    const Group* grp = a.plan.groups + ch.first_group;
-    const int32_t expert = grp[0].expert;
-    const uint8_t* xrow[TT];
-    const uint8_t* xsrow[TT];
-    bool live[TT];
-#pragma unroll
-    for (int tt = 0; tt < TT; ++tt) {
-        const int32_t row = tt < ch.groups ? grp[tt].input_rows[r] : -1;
-        live[tt] = row >= 0;
-        xrow[tt] = (live[tt] ? a.x + size_t(row) * a.x_pitch : a.zero_row) + g * 16;
-        xsrow[tt] = live[tt] ? a.xs + size_t(row) * a.xs_pitch : a.unit_scales;
-    }
-    const uint8_t* img = a.prepared + uint64_t(expert) * a.lay.bytes();
-    const uint8_t* wp = img + a.lay.w13() + uint64_t(cb) * (32 * 4096) + lane * 16;
-    const uint8_t* sp = img + a.lay.s13() + uint64_t(cb) * (8 * 1024) + lane * 4;
-    v4f acc[4][TT];
-#pragma unroll
-    for (int t = 0; t < 4; ++t)
-#pragma unroll
-        for (int tt = 0; tt < TT; ++tt) acc[t][tt] = v4f{0.f, 0.f, 0.f, 0.f};
-    uint32_t bad = 0;
-    gemm_chunk<TT>(acc, wp, sp, 32, int(cb & 7), xrow, xsrow, lane, bad);
     bad |= __shfl_xor(bad, 16);
     bad |= __shfl_xor(bad, 32);
 
@@ -481,6 +487,7 @@ __device__ __forceinline__ void fc1_body(const Fc1Args& a, const Chunk ch, uint3
                 h[t2][i] = silu_up(acc[t2][tt][i], acc[t2 + 2][tt][i]);
                 const uint32_t m = __float_as_uint(h[t2][i]) & 0x7fffffffu;
                 amax = m > amax ? m : amax;
+                __builtin_amdgcn_sched_barrier(0);  // one activation at a time: bounds live registers
             }
         uint32_t o = __shfl_xor(amax, 16);
         amax = o > amax ? o : amax;
@@ -526,6 +533,35 @@ __device__ __forceinline__ void fc1_body(const Fc1Args& a, const Chunk ch, uint3
     }
 }
 
+// One wave's share of FC1 for a chunk of TT groups: 32 intermediate columns x 16*TT rows.
+template <int TT>
+__device__ __forceinline__ void fc1_body(const Fc1Args& a, const Chunk ch, uint32_t cb, uint32_t lane) {
+    const uint32_t r = lane & 15, g = lane >> 4;
+    const Group* grp = a.plan.groups + ch.first_group;
+    const int32_t expert = grp[0].expert;
+    const uint8_t* xrow[TT];
+    const uint8_t* xsrow[TT];
+    bool live[TT];
+#pragma unroll
+    for (int tt = 0; tt < TT; ++tt) {
+        const int32_t row = tt < ch.groups ? grp[tt].input_rows[r] : -1;
+        live[tt] = row >= 0;
+        xrow[tt] = (live[tt] ? a.x + size_t(row) * a.x_pitch : a.zero_row) + g * 16;
+        xsrow[tt] = live[tt] ? a.xs + size_t(row) * a.xs_pitch : a.unit_scales;
+    }
+    const uint8_t* img = a.prepared + uint64_t(expert) * a.lay.bytes();
+    const uint8_t* wp = img + a.lay.w13() + uint64_t(cb) * (32 * 4096) + lane * 16;
+    const uint8_t* sp = img + a.lay.s13() + uint64_t(cb) * (8 * 1024) + lane * 4;
+    v4f acc[4][TT];
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+        for (int tt = 0; tt < TT; ++tt) acc[t][tt] = v4f{0.f, 0.f, 0.f, 0.f};
+    uint32_t bad = 0;
+    gemm_chunk<TT>(acc, wp, sp, 32, 0, xrow, xsrow, lane, bad);
+    fc1_finish<TT>(a, ch, cb, lane, acc, bad, live);
+}
+
 // Stages 2+3: gate/up grouped GEMM, SwiGLU and the v1 requantisation of the intermediate.
 // grid (I/128, chunk capacity), 256 threads; each wave owns one 32-column K32 block of the
 // intermediate for every row of its chunk, so a quantizer block never leaves the wave. A chunk
@@ -560,6 +596,23 @@ struct Fc2Args {
     uint32_t routes;
 };
 
+// FC2 epilogue of one wave: unweighted FP32 rows back to y[original route].
+template <int TT>
+__device__ __forceinline__ void fc2_finish(const Fc2Args& a, uint32_t ob, uint32_t lane, v4f (&acc)[4][TT],
+                                           const int32_t (&route)[TT]) {
+    const uint32_t g = lane >> 4;
+    bool lost = false;
+#pragma unroll
+    for (int tt = 0; tt < TT; ++tt) {
+        if (route[tt] < 0) continue;
+        if (uint32_t(route[tt]) >= a.routes) { lost = true; continue; }
+        float* dst = a.y + size_t(route[tt]) * kHidden + ob * 64 + 4 * g;
+#pragma unroll
+        for (int t = 0; t < 4; ++t) *reinterpret_cast<v4f*>(dst + 16 * t) = acc[t][tt];
+    }
+    if (lost) atomicOr(&a.plan.meta[kFc2Fault], 5u);
+}
+
 // One wave's share of FC2 for a chunk of TT groups: 64 output columns x 16*TT rows.
 template <int TT>
 __device__ __forceinline__ void fc2_body(const Fc2Args& a, const Chunk ch, uint32_t ob, uint32_t lane) {
@@ -587,17 +640,8 @@ __device__ __forceinline__ void fc2_body(const Fc2Args& a, const Chunk ch, uint3
 #pragma unroll
         for (int tt = 0; tt < TT; ++tt) acc[t][tt] = v4f{0.f, 0.f, 0.f, 0.f};
     uint32_t bad = 0;
-    gemm_chunk<TT>(acc, wp, sp, int(ksteps), int(ob % (ksteps / 4)), xrow, xsrow, lane, bad);
-    bool lost = false;
-#pragma unroll
-    for (int tt = 0; tt < TT; ++tt) {
-        if (route[tt] < 0) continue;
-        if (uint32_t(route[tt]) >= a.routes) { lost = true; continue; }
-        float* dst = a.y + size_t(route[tt]) * kHidden + ob * 64 + 4 * g;
-#pragma unroll
-        for (int t = 0; t < 4; ++t) *reinterpret_cast<v4f*>(dst + 16 * t) = acc[t][tt];
-    }
-    if (lost) atomicOr(&a.plan.meta[kFc2Fault], 5u);
+    gemm_chunk<TT>(acc, wp, sp, int(ksteps), 0, xrow, xsrow, lane, bad);
+    fc2_finish<TT>(a, ob, lane, acc, route);
 }
 
 // Stage 4a: down grouped GEMM on the requantised intermediate; rows go back to y[original route].
