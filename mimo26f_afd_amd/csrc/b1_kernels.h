@@ -463,73 +463,89 @@ struct Fc1Args {
     float* tap_gate;          // optional FP32 taps [groups*16][I]
     float* tap_up;
     float* tap_h;
+    // Tile schedule only: per-chunk activation scales in MFMA lane order, [chunk][K/512][8 tiles][64 lanes]
+    // dwords whose byte b is the scale of k-block 4*(4q+b) + lane/16 of row lane%16.
+    const uint8_t* xg;     // FC1 input scales, gathered by gather_scales_kernel
+    const uint32_t* rowbad;  // [chunk][16]: nonzero where a row index of the chunk met an illegal input scale
+    uint8_t* dg;           // the intermediate's scales in the same order, written here for FC2
 };
 
-// FC1 epilogue of one wave: SwiGLU on the gate/up accumulators, then quantizer v1 of each row's
-// 32-column block straight from registers (amax across the four lanes that share a row, frexp-rule
-// exponent, exact-grid RNE, reconstruction check), packed stores of payload and scale.
+// FC1 epilogue of one wave for one activation tile: SwiGLU on the gate/up accumulators (tiles 0,1
+// gate, 2,3 up), then quantizer v1 of each row's 32-column block straight from registers (amax across
+// the four lanes that share a row, frexp-rule exponent, exact-grid RNE, reconstruction check), packed
+// stores of payload and scale. `bad` must already be uniform over the four lanes of a row. dg_chunk,
+// when given, also receives the scale byte in the order FC2's tile schedule reads (see Fc1Args::dg).
+__device__ __forceinline__ void fc1_finish_tile(const Fc1Args& a, const Chunk ch, uint32_t cb, uint32_t lane, int tt,
+                                                const v4f (&acc)[4], uint32_t bad, bool live, uint8_t* dg_chunk) {
+    uint32_t* meta = a.plan.meta;
+    const uint32_t r = lane & 15, g = lane >> 4, I = a.lay.inter;
+    float h[2][4];
+    uint32_t amax = 0;
+#pragma unroll
+    for (int t2 = 0; t2 < 2; ++t2)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            h[t2][i] = silu_up(acc[t2][i], acc[t2 + 2][i]);
+            const uint32_t m = __float_as_uint(h[t2][i]) & 0x7fffffffu;
+            amax = m > amax ? m : amax;
+            __builtin_amdgcn_sched_barrier(0);  // one activation at a time: bounds live registers
+        }
+    uint32_t o = __shfl_xor(amax, 16);
+    amax = o > amax ? o : amax;
+    o = __shfl_xor(amax, 32);
+    amax = o > amax ? o : amax;
+    const size_t grow = size_t(ch.first_group + tt) * 16 + r;
+    const size_t col = size_t(cb) * 32 + 4 * g;
+    if (live && a.tap_h) {
+#pragma unroll
+        for (int t2 = 0; t2 < 2; ++t2) {
+            *reinterpret_cast<v4f*>(a.tap_gate + grow * I + col + 16 * t2) = acc[t2];
+            *reinterpret_cast<v4f*>(a.tap_up + grow * I + col + 16 * t2) = acc[t2 + 2];
+            *reinterpret_cast<v4f*>(a.tap_h + grow * I + col + 16 * t2) = v4f{h[t2][0], h[t2][1], h[t2][2], h[t2][3]};
+        }
+    }
+    const uint32_t block = uint32_t(grow * (I / 32) + cb);
+    uint32_t fault = (amax >= 0x7f800000u || bad) ? 1u : 0u;
+    const int k = quant_scale_exponent(amax);
+    uint32_t word[2] = {0, 0};
+    uint32_t over = 0;
+#pragma unroll
+    for (int t2 = 0; t2 < 2; ++t2)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const uint32_t code = quant_code(__float_as_uint(h[t2][i]), k);
+            over |= quant_reconstructs(code, k) ? 0u : 1u;
+            word[t2] |= code << (8 * i);
+        }
+    over |= __shfl_xor(over, 16);
+    over |= __shfl_xor(over, 32);
+    if (!fault && over) fault = 2;
+    if (!live) return;
+    if (fault) {
+        if (g == 0) {
+            atomicOr(&meta[kQuantFault], fault);
+            atomicMin(&meta[kQuantWhere], block);
+        }
+        return;  // a faulting block publishes no bytes
+    }
+    *reinterpret_cast<uint32_t*>(a.dq + grow * I + col) = word[0];
+    *reinterpret_cast<uint32_t*>(a.dq + grow * I + col + 16) = word[1];
+    if (g == 0) {
+        a.dqs[grow * (I / 32) + cb] = uint8_t(k + 127);
+        // Block cb is k-block cb of FC2: k-step cb/4, lane group cb%4.
+        if (dg_chunk) dg_chunk[((((cb >> 4) * 8 + tt) * 64 + (cb & 3) * 16 + r) << 2) + ((cb >> 2) & 3)] = uint8_t(k + 127);
+    }
+}
+
 template <int TT>
 __device__ __forceinline__ void fc1_finish(const Fc1Args& a, const Chunk ch, uint32_t cb, uint32_t lane,
                                            v4f (&acc)[4][TT], uint32_t bad, const bool (&live)[TT]) {
-    uint32_t* meta = a.plan.meta;
-    const uint32_t r = lane & 15, g = lane >> 4, I = a.lay.inter;
     bad |= __shfl_xor(bad, 16);
     bad |= __shfl_xor(bad, 32);
-
 #pragma unroll
     for (int tt = 0; tt < TT; ++tt) {
-        float h[2][4];
-        uint32_t amax = 0;
-#pragma unroll
-        for (int t2 = 0; t2 < 2; ++t2)
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                h[t2][i] = silu_up(acc[t2][tt][i], acc[t2 + 2][tt][i]);
-                const uint32_t m = __float_as_uint(h[t2][i]) & 0x7fffffffu;
-                amax = m > amax ? m : amax;
-                __builtin_amdgcn_sched_barrier(0);  // one activation at a time: bounds live registers
-            }
-        uint32_t o = __shfl_xor(amax, 16);
-        amax = o > amax ? o : amax;
-        o = __shfl_xor(amax, 32);
-        amax = o > amax ? o : amax;
-        const size_t grow = size_t(ch.first_group + tt) * 16 + r;
-        const size_t col = size_t(cb) * 32 + 4 * g;
-        if (live[tt] && a.tap_h) {
-#pragma unroll
-            for (int t2 = 0; t2 < 2; ++t2) {
-                *reinterpret_cast<v4f*>(a.tap_gate + grow * I + col + 16 * t2) = acc[t2][tt];
-                *reinterpret_cast<v4f*>(a.tap_up + grow * I + col + 16 * t2) = acc[t2 + 2][tt];
-                *reinterpret_cast<v4f*>(a.tap_h + grow * I + col + 16 * t2) = v4f{h[t2][0], h[t2][1], h[t2][2], h[t2][3]};
-            }
-        }
-        const uint32_t block = uint32_t(grow * (I / 32) + cb);
-        uint32_t fault = (amax >= 0x7f800000u || bad) ? 1u : 0u;
-        const int k = quant_scale_exponent(amax);
-        uint32_t word[2] = {0, 0};
-        uint32_t over = 0;
-#pragma unroll
-        for (int t2 = 0; t2 < 2; ++t2)
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const uint32_t code = quant_code(__float_as_uint(h[t2][i]), k);
-                over |= quant_reconstructs(code, k) ? 0u : 1u;
-                word[t2] |= code << (8 * i);
-            }
-        over |= __shfl_xor(over, 16);
-        over |= __shfl_xor(over, 32);
-        if (!fault && over) fault = 2;
-        if (!live[tt]) continue;
-        if (fault) {
-            if (g == 0) {
-                atomicOr(&meta[kQuantFault], fault);
-                atomicMin(&meta[kQuantWhere], block);
-            }
-            continue;  // a faulting block publishes no bytes
-        }
-        *reinterpret_cast<uint32_t*>(a.dq + grow * I + col) = word[0];
-        *reinterpret_cast<uint32_t*>(a.dq + grow * I + col + 16) = word[1];
-        if (g == 0) a.dqs[grow * (I / 32) + cb] = uint8_t(k + 127);
+        const v4f tile[4] = {acc[0][tt], acc[1][tt], acc[2][tt], acc[3][tt]};
+        fc1_finish_tile(a, ch, cb, lane, tt, tile, bad, live[tt], nullptr);
     }
 }
 
@@ -594,6 +610,7 @@ struct Fc2Args {
     const uint8_t* unit_scales;
     float* y;         // [routes][4096], original (token, slot) order, unweighted
     uint32_t routes;
+    const uint8_t* dg;  // tile schedule only: the intermediate's scales in MFMA lane order (see Fc1Args)
 };
 
 // FC2 epilogue of one wave: unweighted FP32 rows back to y[original route].

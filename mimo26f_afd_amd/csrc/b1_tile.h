@@ -1,18 +1,27 @@
-// Prefill-size schedule of FC1 / FC2: four waves per workgroup, one per SIMD, each holding a
-// 128-row x (16*TT)-row accumulator block (eight weight tiles x TT activation tiles, up to 256
-// accumulator registers). Operands travel global -> LDS with the direct-to-LDS loads of gfx950
-// (no staging registers, so the prefetch depth is paid in LDS, not in VGPRs), always two k-steps
-// ahead of the MFMAs that consume them: every wave streams its own weight fragments into a private
-// two-stage ring (a stage is free once its fragments sit in registers), and the chunk's activation
-// tiles are staged once per workgroup in a three-stage ring shared by the four waves, so each
-// activation byte leaves L2 once per 256 (FC1) or 512 (FC2) output columns.
+// Prefill-size schedule of FC1 / FC2: workgroups of four waves, two workgroups per compute unit.
+//
+// A wave accumulates one column block (four weight tiles: 32 intermediate columns of FC1, 64 output
+// columns of FC2) against all TT activation tiles of its chunk: 4*TT accumulator tiles, 128
+// accumulation registers at TT = 8, which leaves the other half of the register file to a second
+// workgroup on the same SIMDs. That second workgroup is what hides everything that is not an MFMA:
+// while one workgroup looks up its chunk, waits for its first operands or runs its epilogue
+// (SwiGLU + requantisation, or the FP32 row stores), the other one multiplies.
+//
+// Operands travel global -> LDS with the direct-to-LDS loads of gfx950 (no staging registers, so the
+// prefetch depth is paid in LDS, not in VGPRs), always two k-steps ahead of the MFMAs that consume
+// them: every wave streams its own weight fragments into a private two-stage ring (a stage is free
+// once its fragments sit in registers), and the chunk's activation tiles are staged once per
+// workgroup in a three-stage ring shared by the four waves. Scales never touch LDS: weight scales
+// are stored in MFMA lane order by the one-time preparation, and activation scales are brought into
+// the same order per chunk (gather_scales_kernel for the caller's rows, the FC1 epilogue for the
+// intermediate), so one dword per lane carries the scale bytes of four k-steps and the MFMA picks
+// its byte with op_sel.
 //
 // Reference counterparts: fc1_m64 / fc2_m64, the weight-reuse chunk kernels of
 // crates/mimo26-spark/kernels/b1_fc1_m64.cuh:111-205,378-491 (cp.async multi-stage staging there).
 //
-// LDS, dynamic:  [4 waves][2 stages][8 tiles][64 lanes][16 B]   weight fragments (private per wave)
-//                [3 stages][TT tiles][2 halves][64 lanes][16 B] activation fragments (shared)
-//                [TT tiles][ksteps][16 rows][4 B]               activation scale bytes of the chunk
+// LDS, dynamic, 80 KB:  [4 waves][2 stages][4 tiles][64 lanes][16 B]   weight fragments (private per wave)
+//                       [3 stages][8 tiles][2 halves][64 lanes][16 B]  activation fragments (shared)
 // All fragment cells sit in MFMA lane order, so one direct load fills a 1 KB cell row and one
 // ds_read_b128 per lane reads it back without bank conflicts. The compiler does not order LDS reads
 // against direct-to-LDS loads; the vmcnt waits below do, and rely on the issue order stated there.
@@ -25,10 +34,10 @@
 namespace m26g {
 
 constexpr int kTileThreads = 256, kTileWaves = 4, kWeightStages = 2, kActStages = 3;
-
-__host__ __device__ constexpr uint32_t tile_lds_bytes(int tt, uint32_t k) {
-    return uint32_t(kTileWaves) * kWeightStages * 8192 + uint32_t(kActStages) * tt * 2048 + (k / 128) * tt * 64;
-}
+constexpr uint32_t kTileLdsBytes = kTileWaves * kWeightStages * 4096 + kActStages * 8 * 2048;
+static_assert(kTileLdsBytes == 80 * 1024, "two workgroups share the 160 KB of a compute unit");
+// Bytes of one chunk's gathered activation scales for a K-deep product: [K/512][8][64] dwords.
+__host__ __device__ constexpr uint32_t gathered_scale_bytes(uint32_t k) { return (k / 512) * 2048; }
 
 typedef __attribute__((address_space(3))) void* lds_ptr;
 typedef const __attribute__((address_space(1))) void* global_ptr;
@@ -44,264 +53,331 @@ template <int N> __device__ __forceinline__ void wait_loads_but() {
 // LDS-only workgroup barrier: outstanding global prefetches stay in flight across it.
 __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
-// acc += A(FP4, scale byte SEL of sa) x B(FP8, scale byte 0 of sb), in place. Written as an
-// instruction so destination and addend are the same registers: left to the compiler, a third of
-// these MFMAs get a different destination and the loop drowns in accumulator copies. Half of a
-// wave's accumulators are pinned to accumulation registers and half to vector registers, which
-// leaves the other half of the accumulation file to the register allocator as spill space.
-#define M26G_MFMA(sel_text, cons)                                                                              \
+// acc += A(FP4, scale byte SEL of sa) x B(FP8, scale byte SEL of sb), in place, accumulator pinned
+// to the accumulation registers. Written as an instruction so destination and addend are the same
+// registers: left to the compiler, a third of these MFMAs get a different destination and the loop
+// drowns in accumulator copies.
+#define M26G_MFMA(sel_text)                                                                                    \
     asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 %0, %1, %2, %0, %3, %4 " sel_text " cbsz:4"                  \
-                 : cons(acc) : "v"(a), "v"(b), "v"(sa), "v"(sb))
-template <int SEL, bool AGPR>
+                 : "+a"(acc) : "v"(a), "v"(b), "v"(sa), "v"(sb))
+template <int SEL>
 __device__ __forceinline__ void mfma_acc(v4f& acc, const v4i& a, const v8i& b, uint32_t sa, uint32_t sb) {
-    if constexpr (AGPR) {
-        if constexpr (SEL == 0) M26G_MFMA("op_sel_hi:[0,0,0]", "+a");
-        else if constexpr (SEL == 1) M26G_MFMA("op_sel:[1,0,0] op_sel_hi:[0,0,0]", "+a");
-        else if constexpr (SEL == 2) M26G_MFMA("op_sel_hi:[1,0,0]", "+a");
-        else M26G_MFMA("op_sel:[1,0,0] op_sel_hi:[1,0,0]", "+a");
-    } else {
-        if constexpr (SEL == 0) M26G_MFMA("op_sel_hi:[0,0,0]", "+v");
-        else if constexpr (SEL == 1) M26G_MFMA("op_sel:[1,0,0] op_sel_hi:[0,0,0]", "+v");
-        else if constexpr (SEL == 2) M26G_MFMA("op_sel_hi:[1,0,0]", "+v");
-        else M26G_MFMA("op_sel:[1,0,0] op_sel_hi:[1,0,0]", "+v");
-    }
+    if constexpr (SEL == 0) M26G_MFMA("op_sel_hi:[0,0,0]");
+    else if constexpr (SEL == 1) M26G_MFMA("op_sel:[1,1,0] op_sel_hi:[0,0,0]");
+    else if constexpr (SEL == 2) M26G_MFMA("op_sel_hi:[1,1,0]");
+    else M26G_MFMA("op_sel:[1,1,0] op_sel_hi:[1,1,0]");
 }
 #undef M26G_MFMA
 
-// One workgroup's GEMM for a chunk. Wave `wv` accumulates eight weight tiles (two 4-tile blocks at
-// wp0 / wp1, scales sp0 / sp1) against all TT activation tiles. The wave stages TT/4 activation
-// tiles per k-step: `row[i]` / `srow[i]` are this lane's row of tile wv*(TT/4)+i (lane offset
-// 16*(lane/16) included), so the lane that loads a fragment cell is the lane that will hold it.
+// Rewrites the activation scale rows of every chunk into MFMA lane order (layout at Fc1Args::xg) and
+// checks them against the legal window [105, 247] (crates/mimo26-expert/kernels/b1/grouped.cu:28,37
+// holds the reference's check). Padded rows get the unit scale 127. rowbad[chunk][r] collects the
+// verdict of row r of all tiles, the granularity the FC1 epilogue reports faults at.
+// grid (chunk capacity), 256 threads = 8 tiles x 16 rows x 2 halves of a scale row.
+__global__ void __launch_bounds__(256) gather_scales_kernel(PlanView plan, const uint8_t* __restrict__ xs, size_t xs_pitch,
+                                                            uint32_t* __restrict__ xg, uint32_t* __restrict__ rowbad) {
+    __shared__ uint32_t flags[16];
+    const uint32_t c = blockIdx.x, tid = threadIdx.x;
+    if (plan.meta[kPlanFault] || c >= plan.meta[kChunkCount]) return;
+    const Chunk ch = plan.chunks[c];
+    if (ch.groups < 1 || ch.groups > 8) return;  // FC1 reports the broken chunk
+    const uint32_t tt = tid >> 5, r = (tid >> 1) & 15, half = tid & 1;
+    if (tid < 16) flags[tid] = 0;
+    __syncthreads();
+    const int32_t row = int32_t(tt) < ch.groups ? plan.groups[ch.first_group + tt].input_rows[r] : -1;
+    uint32_t bad = 0;
+#pragma unroll
+    for (uint32_t j = 0; j < 4; ++j) {
+        const uint32_t q = 4 * half + j;
+        uint32_t in[4] = {0x7f7f7f7fu, 0x7f7f7f7fu, 0x7f7f7f7fu, 0x7f7f7f7fu};
+        if (row >= 0) {
+            const uint8_t* src = xs + size_t(row) * xs_pitch + 16 * q;
+#pragma unroll
+            for (uint32_t b = 0; b < 4; ++b)
+                in[b] = uint32_t(src[4 * b]) | uint32_t(src[4 * b + 1]) << 8 | uint32_t(src[4 * b + 2]) << 16 |
+                        uint32_t(src[4 * b + 3]) << 24;
+        }
+#pragma unroll
+        for (uint32_t g = 0; g < 4; ++g) {
+            uint32_t out = 0;
+#pragma unroll
+            for (uint32_t b = 0; b < 4; ++b) {
+                const uint32_t s = (in[b] >> (8 * g)) & 0xffu;
+                bad |= (s - 105u) > 142u ? 1u : 0u;
+                out |= s << (8 * b);
+            }
+            xg[((size_t(c) * (kHidden / 512) + q) * 8 + tt) * 64 + g * 16 + r] = out;
+        }
+    }
+    if (bad) atomicOr(&flags[r], 1u);
+    __syncthreads();
+    if (tid < 16) rowbad[c * 16 + tid] = flags[tid];
+}
+
+// One wave's GEMM for a chunk: four weight tiles (fragments at wp, scale dwords at sp, both with the
+// lane offset included) against TT activation tiles. The wave stages TT/4 of the activation tiles
+// per k-step: `row[i]` is this lane's row of tile wv*(TT/4)+i (lane offset 16*(lane/16) included),
+// so the lane that loads a fragment cell is the lane that will hold it. `sx` points at this lane's
+// dword of tile 0, quad 0 of the chunk's gathered activation scales.
 template <int TT>
-__device__ __forceinline__ void gemm_chunk_lds(v4f (&acc0)[4][TT], v4f (&acc1)[4][TT], const uint8_t* __restrict__ wp0,
-                                               const uint8_t* __restrict__ wp1, const uint8_t* __restrict__ sp0,
-                                               const uint8_t* __restrict__ sp1, int ksteps,
-                                               const uint8_t* const (&row)[TT / 4], const uint8_t* const (&srow)[TT / 4],
-                                               uint32_t wv, uint32_t lane, uint8_t* lds, uint32_t& bad) {
+__device__ __forceinline__ void gemm_chunk_lds(v4f (&acc)[4][TT], const uint8_t* __restrict__ wp,
+                                               const uint8_t* __restrict__ sp, const uint8_t* __restrict__ sx, int ksteps,
+                                               const uint8_t* const (&row)[TT / 4], uint32_t wv, uint32_t lane, uint8_t* lds) {
     static_assert(TT == 4 || TT == 8, "activation tiles per chunk");
     constexpr int kMine = TT / kTileWaves;  // activation tiles this wave stages
-    const uint32_t r = lane & 15, g = lane >> 4;
-    uint8_t* wring = lds + wv * (kWeightStages * 8192);                 // [stage][tile][lane][16]
-    uint8_t* aring = lds + kTileWaves * kWeightStages * 8192;           // [stage][tt][half][lane][16]
-    uint8_t* stab = aring + kActStages * TT * 2048;                     // [tt][ks][r][4]
-    // The chunk's activation scale bytes, [tt][ks][row] dwords: one direct load moves the dwords of four
-    // k-steps x 16 rows (lane = 16*j + row fetches k-step 4*i + j of its row).
-#pragma unroll
-    for (int m = 0; m < kMine; ++m)
-        for (int i = 0; i < ksteps / 4; ++i)
-            __builtin_amdgcn_global_load_lds((global_ptr)(srow[m] + (4 * i + g) * 4),
-                                             (lds_ptr)(stab + ((wv * kMine + m) * ksteps + 4 * i) * 64), 4, 0, 0);
+    uint8_t* wring = lds + wv * (kWeightStages * 4096);          // [stage][tile][lane][16]
+    uint8_t* aring = lds + kTileWaves * kWeightStages * 4096;    // [stage][tt][half][lane][16]
     // The direct loads of one k-step: item i < 2*kMine is an activation cell (tile i/2, half i%2),
-    // the other eight are the weight rows. A k-step issues exactly kPerStep of them, spread over its
+    // the other four are the weight rows. A k-step issues exactly kPerStep of them, spread over its
     // TT groups of MFMAs so the memory pipeline never sees a burst; the waits count on that total.
-    constexpr int kPerStep = 2 * kMine + 8;
+    constexpr int kPerStep = 2 * kMine + 4;
     auto stage_item = [&](int item, int ks, uint32_t astage, uint32_t wstage) {
         if (item < 2 * kMine) {
             const int m = item >> 1, half = item & 1;
             load_row_to_lds(row[m] + ks * 128 + half * 64, aring + ((astage * TT + wv * kMine + m) * 2 + half) * 1024);
         } else {
             const int t = item - 2 * kMine;
-            load_row_to_lds((t < 4 ? wp0 : wp1) + size_t(ks) * 4096 + (t & 3) * 1024, wring + wstage * 8192 + t * 1024);
+            load_row_to_lds(wp + size_t(ks) * 4096 + t * 1024, wring + wstage * 4096 + t * 1024);
         }
     };
     auto stage_all = [&](int ks, uint32_t astage, uint32_t wstage) {
 #pragma unroll
         for (int item = 0; item < kPerStep; ++item) stage_item(item, ks, astage, wstage);
     };
-    v4i af[2][8];  // weight fragments of this k-step and the next
-    auto read_weights = [&](v4i (&a)[8], uint32_t stage) {
+    v4i af[2][4];  // weight fragments of this k-step and the next
+    auto read_weights = [&](v4i (&a)[4], uint32_t stage) {
 #pragma unroll
-        for (int t = 0; t < 8; ++t) a[t] = *reinterpret_cast<const v4i*>(wring + stage * 8192 + t * 1024 + lane * 16);
+        for (int t = 0; t < 4; ++t) a[t] = *reinterpret_cast<const v4i*>(wring + stage * 4096 + t * 1024 + lane * 16);
     };
-    const int last = ksteps - 1;
+    // Scale dwords of a quad of k-steps (four weight tiles, TT activation tiles), in two register sets
+    // that alternate. They are loaded by hand a whole quad ahead: a load the compiler knows of makes
+    // it drain every outstanding load, the direct ones included, before the first use. The compiler
+    // takes these registers for loaded the moment the instruction issues, so nothing but the MFMAs
+    // may read them, and those sit behind the vmcnt waits of the quad before.
+    uint32_t sw0[4], sa0[TT], sw1[4], sa1[TT];
+    auto load_scales = [&](uint32_t (&w)[4], uint32_t (&x)[TT], int q) {
+        const uint8_t* pw = sp + size_t(q) * 1024;
+        const uint8_t* px = sx + size_t(q) * 2048;
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+            asm volatile("global_load_dword %0, %1, off offset:%2" : "=v"(w[t]) : "v"(pw), "n"(t * 256) : "memory");
+#pragma unroll
+        for (int tt = 0; tt < TT; ++tt)
+            asm volatile("global_load_dword %0, %1, off offset:%2" : "=v"(x[tt]) : "v"(px), "n"(tt * 256) : "memory");
+    };
+    const int last = ksteps - 1, quads = ksteps / 4;
+    load_scales(sw0, sa0, 0);
     stage_all(0, 0, 0);
     stage_all(1 < last ? 1 : last, 1, 1);
-    wait_loads_but<kPerStep>();  // step 0 has landed, step 1 may still fly
+    wait_loads_but<kPerStep>();  // step 0 and the first scales have landed, step 1 may still fly
     read_weights(af[0], 0);
     lds_barrier();
-    uint32_t wr = 0, ar = 0;  // weight stage holding step k+... see below; activation stage of step k
-#pragma unroll 1
-    for (int q = 0; q < ksteps / 4; ++q) {
-        uint32_t sw[8];
-#pragma unroll
-        for (int t = 0; t < 4; ++t) {
-            sw[t] = *reinterpret_cast<const uint32_t*>(sp0 + size_t(q) * 1024 + t * 256);
-            sw[4 + t] = *reinterpret_cast<const uint32_t*>(sp1 + size_t(q) * 1024 + t * 256);
-        }
-        // One k-step with MFMA scale select b = ks % 4 (an immediate, hence the macro).
-#define M26G_KSTEP(b)                                                                                          \
-        {                                                                                                      \
-            const int ks = 4 * q + (b);                                                                        \
-            /* Weights of step k sit in registers, so their stage `wr` takes step k+2; step k+1 is in     */  \
-            /* stage wr^1. Activations: step k reads stage ar, k+1 sits in ar+1, k+2 goes to ar+2.        */  \
-            const uint32_t ar1 = ar == kActStages - 1 ? 0 : ar + 1, ar2 = ar1 == kActStages - 1 ? 0 : ar1 + 1; \
-            /* Past the end the last step is staged again into stages nobody reads any more. */               \
-            const int ahead = ks + 2 < last ? ks + 2 : last;                                                   \
-            const uint8_t* fs = aring + ar * TT * 2048 + lane * 16;                                            \
-            const uint8_t* ss = stab + (ks * 16 + r) * 4 + g;                                                  \
-            v4i lo = *reinterpret_cast<const v4i*>(fs), hi = *reinterpret_cast<const v4i*>(fs + 1024);         \
-            uint32_t s = ss[0];                                                                                \
-            __builtin_amdgcn_sched_barrier(0);                                                                 \
-            _Pragma("unroll") for (int tt = 0; tt < TT; ++tt) {                                                \
-                _Pragma("unroll") for (int item = 0; item < kPerStep; ++item)                                  \
-                    if (item * TT / kPerStep == tt) stage_item(item, ahead, ar2, wr);                          \
-                const v8i bv = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};                               \
-                const uint32_t sc = s;                                                                         \
-                bad |= (sc - 105u) > 142u ? 1u : 0u; /* activation scales are legal only in [105, 247] */      \
-                if (tt + 1 < TT) { /* the next fragment is on its way while this one multiplies */             \
-                    lo = *reinterpret_cast<const v4i*>(fs + (tt + 1) * 2048);                                  \
-                    hi = *reinterpret_cast<const v4i*>(fs + (tt + 1) * 2048 + 1024);                           \
-                    s = ss[(tt + 1) * ksteps * 64];                                                            \
-                } else {                                                                                       \
-                    /* Everything but this step's own loads (step k+2) has landed: activations and */          \
-                    /* weights of step k+1, issued one whole k-step ago.                            */          \
-                    wait_loads_but<kPerStep>();                                                                \
-                    read_weights(af[((b) + 1) & 1], wr ^ 1);                                                   \
-                }                                                                                              \
-                __builtin_amdgcn_sched_barrier(0);                                                             \
-                _Pragma("unroll") for (int t = 0; t < 4; ++t)                                                  \
-                    mfma_acc<(b), true>(acc0[t][tt], af[(b) & 1][t], bv, sw[t], sc);                            \
-                _Pragma("unroll") for (int t = 0; t < 4; ++t)                                                  \
-                    mfma_acc<(b), false>(acc1[t][tt], af[(b) & 1][4 + t], bv, sw[4 + t], sc);                    \
-                __builtin_amdgcn_sched_barrier(0);                                                             \
+    uint32_t wr = 0, ar = 0;  // weight stage that takes step k+2; activation stage of step k
+    int q = 0;
+    // One k-step with MFMA scale select b = ks % 4 (an immediate, hence the macro).
+#define M26G_KSTEP(b, SW, SA)                                                                                  \
+    {                                                                                                          \
+        const int ks = 4 * q + (b);                                                                            \
+        /* Weights of step k sit in registers, so their stage `wr` takes step k+2; step k+1 is in     */      \
+        /* stage wr^1. Activations: step k reads stage ar, k+1 sits in ar+1, k+2 goes to ar+2.        */      \
+        const uint32_t ar1 = ar == kActStages - 1 ? 0 : ar + 1, ar2 = ar1 == kActStages - 1 ? 0 : ar1 + 1;     \
+        /* Past the end the last step is staged again into stages nobody reads any more. */                   \
+        const int ahead = ks + 2 < last ? ks + 2 : last;                                                       \
+        const uint8_t* fs = aring + ar * TT * 2048 + lane * 16;                                                \
+        v4i lo = *reinterpret_cast<const v4i*>(fs), hi = *reinterpret_cast<const v4i*>(fs + 1024);             \
+        __builtin_amdgcn_sched_barrier(0);                                                                     \
+        _Pragma("unroll") for (int tt = 0; tt < TT; ++tt) {                                                    \
+            _Pragma("unroll") for (int item = 0; item < kPerStep; ++item)                                      \
+                if (item * TT / kPerStep == tt) stage_item(item, ahead, ar2, wr);                              \
+            const v8i bv = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};                                   \
+            if (tt + 1 < TT) { /* the next fragment is on its way while this one multiplies */                 \
+                lo = *reinterpret_cast<const v4i*>(fs + (tt + 1) * 2048);                                      \
+                hi = *reinterpret_cast<const v4i*>(fs + (tt + 1) * 2048 + 1024);                               \
+            } else {                                                                                           \
+                /* Everything but this step's own loads (step k+2) has landed: activations and weights */      \
+                /* of step k+1, issued one whole k-step ago, and the next quad's scales, older still.   */      \
+                wait_loads_but<kPerStep>();                                                                    \
+                read_weights(af[((b) + 1) & 1], wr ^ 1);                                                       \
             }                                                                                                  \
-            wr ^= 1;                                                                                           \
-            ar = ar1;                                                                                          \
-            lds_barrier();                                                                                     \
             __builtin_amdgcn_sched_barrier(0);                                                                 \
-        }
-        M26G_KSTEP(0)
-        M26G_KSTEP(1)
-        M26G_KSTEP(2)
-        M26G_KSTEP(3)
-#undef M26G_KSTEP
+            _Pragma("unroll") for (int t = 0; t < 4; ++t)                                                      \
+                mfma_acc<(b)>(acc[t][tt], af[(b) & 1][t], bv, SW[t], SA[tt]);                                   \
+            __builtin_amdgcn_sched_barrier(0);                                                                 \
+        }                                                                                                      \
+        wr ^= 1;                                                                                               \
+        ar = ar1;                                                                                              \
+        lds_barrier();                                                                                         \
+        __builtin_amdgcn_sched_barrier(0);                                                                     \
     }
+    // A quad: fetch the next quad's scales into the other set, then four k-steps on this set.
+#define M26G_QUAD(SW, SA, NW, NA)                                                                              \
+    {                                                                                                          \
+        load_scales(NW, NA, q + 1 < quads ? q + 1 : q);                                                        \
+        __builtin_amdgcn_sched_barrier(0);                                                                     \
+        M26G_KSTEP(0, SW, SA)                                                                                  \
+        M26G_KSTEP(1, SW, SA)                                                                                  \
+        M26G_KSTEP(2, SW, SA)                                                                                  \
+        M26G_KSTEP(3, SW, SA)                                                                                  \
+        ++q;                                                                                                   \
+    }
+#pragma unroll 1
+    while (q + 1 < quads) {
+        M26G_QUAD(sw0, sa0, sw1, sa1)
+        M26G_QUAD(sw1, sa1, sw0, sa0)
+    }
+    if (q < quads) M26G_QUAD(sw0, sa0, sw1, sa1)  // odd count: an even number of quads ends on set 0
+#undef M26G_QUAD
+#undef M26G_KSTEP
     wait_loads_but<0>();  // the re-staged tail loads must land before the LDS is reused or the wave ends
     // The MFMAs above are opaque to the compiler's hazard tracking: let the last ones retire before
     // the epilogue reads the accumulators (8 passes of 4 cycles, plus margin).
     asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15" ::: "memory");
 }
 
-// FC1 for one chunk of up to TT groups by one workgroup: 256 intermediate columns x 16*TT rows.
+// The epilogues index everything by the lane number. Handing them a copy the compiler cannot see
+// through keeps their address arithmetic behind the k-loop, where it would otherwise be hoisted to
+// and held in registers the loop needs.
+__device__ __forceinline__ uint32_t after_loop(uint32_t lane) {
+    asm volatile("" : "+v"(lane));
+    return lane;
+}
+
+// FC1 for chunk c by one workgroup: 128 intermediate columns x 16*TT rows; the wave owns block cb.
 template <int TT>
-__device__ __forceinline__ void fc1_tile_body(const Fc1Args& a, const Chunk ch, uint32_t wv, uint32_t lane, uint8_t* lds) {
+__device__ __forceinline__ void fc1_tile_body(const Fc1Args& a, const Chunk ch, uint32_t c, uint32_t cb, uint32_t wv,
+                                              uint32_t lane, uint8_t* lds) {
     constexpr int kMine = TT / kTileWaves;
-    const uint32_t r = lane & 15, g = lane >> 4, cb0 = blockIdx.x * 8 + wv * 2;
+    const uint32_t r = lane & 15, g = lane >> 4;
     const Group* grp = a.plan.groups + ch.first_group;
     const int32_t expert = grp[0].expert;
     const uint8_t* row[kMine];
-    const uint8_t* srow[kMine];
 #pragma unroll
     for (int m = 0; m < kMine; ++m) {
         const int lt = int(wv) * kMine + m;
         const int32_t mine = lt < ch.groups ? grp[lt].input_rows[r] : -1;
         row[m] = (mine >= 0 ? a.x + size_t(mine) * a.x_pitch : a.zero_row) + g * 16;
-        srow[m] = mine >= 0 ? a.xs + size_t(mine) * a.xs_pitch : a.unit_scales;
     }
     const uint8_t* img = a.prepared + uint64_t(expert) * a.lay.bytes();
-    const uint8_t* wp = img + a.lay.w13() + uint64_t(cb0) * (32 * 4096) + lane * 16;
-    const uint8_t* sp = img + a.lay.s13() + uint64_t(cb0) * (8 * 1024) + lane * 4;
-    v4f acc0[4][TT], acc1[4][TT];
+    const uint8_t* wp = img + a.lay.w13() + uint64_t(cb) * (32 * 4096) + lane * 16;
+    const uint8_t* sp = img + a.lay.s13() + uint64_t(cb) * (8 * 1024) + lane * 4;
+    const uint8_t* sx = a.xg + size_t(c) * gathered_scale_bytes(kHidden) + lane * 4;
+    v4f acc[4][TT];
 #pragma unroll
     for (int t = 0; t < 4; ++t)
 #pragma unroll
-        for (int tt = 0; tt < TT; ++tt) acc0[t][tt] = acc1[t][tt] = v4f{0.f, 0.f, 0.f, 0.f};
-    uint32_t bad = 0;
-    gemm_chunk_lds<TT>(acc0, acc1, wp, wp + 32 * 4096, sp, sp + 8 * 1024, int(kHidden / 128), row, srow, wv, lane, lds, bad);
-    bad |= __shfl_xor(bad, 16);  // a row's four lanes see its four scale bytes of a k-step
-    bad |= __shfl_xor(bad, 32);
-    bool live[TT];  // looked up after the GEMM: nothing extra stays live across the k-loop
+        for (int tt = 0; tt < TT; ++tt) acc[t][tt] = v4f{0.f, 0.f, 0.f, 0.f};
+    gemm_chunk_lds<TT>(acc, wp, sp, sx, int(kHidden / 128), row, wv, lane, lds);
+    const uint32_t lane2 = after_loop(lane), r2 = lane2 & 15;
+    const uint32_t bad = a.rowbad[c * 16 + r2];
+    bool live[TT];
 #pragma unroll
-    for (int tt = 0; tt < TT; ++tt) live[tt] = tt < ch.groups && grp[tt].input_rows[r] >= 0;
-    fc1_finish<TT>(a, ch, cb0, lane, acc0, bad, live);
-    fc1_finish<TT>(a, ch, cb0 + 1, lane, acc1, bad, live);
-}
-
-// FC2 for one chunk by one workgroup: 512 output columns x 16*TT rows.
-template <int TT>
-__device__ __forceinline__ void fc2_tile_body(const Fc2Args& a, const Chunk ch, uint32_t wv, uint32_t lane, uint8_t* lds) {
-    constexpr int kMine = TT / kTileWaves;
-    const uint32_t r = lane & 15, g = lane >> 4, ob0 = blockIdx.x * 8 + wv * 2, I = a.lay.inter;
-    const Group* grp = a.plan.groups + ch.first_group;
-    const int32_t expert = grp[0].expert;
-    int32_t route[TT];
+    for (int tt = 0; tt < TT; ++tt) live[tt] = tt < ch.groups && grp[tt].input_rows[r2] >= 0;
+    // The accumulators leave the accumulation registers through the wave's own, now idle, weight ring:
+    // whole-tile LDS writes keep them out of the register allocator's hands until the very end (element
+    // reads straight from the accumulation file make it split their live ranges across the k-loop).
+    uint8_t* bounce = lds + wv * (kWeightStages * 4096) + lane2 * 16;
+    const uint32_t bounce_at = uint32_t(uintptr_t((lds_ptr)bounce));
+    uint8_t* dg_chunk = a.dg + size_t(c) * gathered_scale_bytes(a.lay.inter);
 #pragma unroll
     for (int tt = 0; tt < TT; ++tt) {
-        const bool live = tt < ch.groups && int32_t(r) < grp[tt].rows;
-        route[tt] = live ? a.plan.original[grp[tt].route_base + r] : -1;
+        const uint32_t slot = (tt & 1) * 4096;
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+            asm volatile("ds_write_b128 %0, %1" ::"v"(bounce_at + slot + t * 1024), "a"(acc[t][tt]) : "memory");
+        v4f tile[4];
+#pragma unroll
+        for (int t = 0; t < 4; ++t) tile[t] = *reinterpret_cast<const v4f*>(bounce + slot + t * 1024);
+        fc1_finish_tile(a, ch, cb, lane2, tt, tile, bad, live[tt], dg_chunk);
     }
+}
+
+// FC2 for chunk c by one workgroup: 256 output columns x 16*TT rows; the wave owns block ob.
+template <int TT>
+__device__ __forceinline__ void fc2_tile_body(const Fc2Args& a, const Chunk ch, uint32_t c, uint32_t ob, uint32_t wv,
+                                              uint32_t lane, uint8_t* lds) {
+    constexpr int kMine = TT / kTileWaves;
+    const uint32_t r = lane & 15, g = lane >> 4, I = a.lay.inter;
+    const Group* grp = a.plan.groups + ch.first_group;
+    const int32_t expert = grp[0].expert;
     const uint8_t* row[kMine];
-    const uint8_t* srow[kMine];
 #pragma unroll
     for (int m = 0; m < kMine; ++m) {
         const int lt = int(wv) * kMine + m;
         const bool mine = lt < ch.groups && int32_t(r) < grp[lt].rows;
         const size_t grow = size_t(ch.first_group + lt) * 16 + r;
         row[m] = (mine ? a.dq + grow * I : a.zero_row) + g * 16;
-        srow[m] = mine ? a.dqs + grow * (I / 32) : a.unit_scales;
     }
     const uint32_t ksteps = I / 128;
     const uint8_t* img = a.prepared + uint64_t(expert) * a.lay.bytes();
-    const uint8_t* wp = img + a.lay.w2() + uint64_t(ob0) * ksteps * 4096 + lane * 16;
-    const uint8_t* sp = img + a.lay.s2() + uint64_t(ob0) * (ksteps / 4) * 1024 + lane * 4;
-    v4f acc0[4][TT], acc1[4][TT];
+    const uint8_t* wp = img + a.lay.w2() + uint64_t(ob) * ksteps * 4096 + lane * 16;
+    const uint8_t* sp = img + a.lay.s2() + uint64_t(ob) * (ksteps / 4) * 1024 + lane * 4;
+    const uint8_t* sx = a.dg + size_t(c) * gathered_scale_bytes(I) + lane * 4;
+    v4f acc[4][TT];
 #pragma unroll
     for (int t = 0; t < 4; ++t)
 #pragma unroll
-        for (int tt = 0; tt < TT; ++tt) acc0[t][tt] = acc1[t][tt] = v4f{0.f, 0.f, 0.f, 0.f};
-    uint32_t bad = 0;
-    gemm_chunk_lds<TT>(acc0, acc1, wp, wp + size_t(ksteps) * 4096, sp, sp + size_t(ksteps / 4) * 1024, int(ksteps), row, srow,
-                       wv, lane, lds, bad);
-    fc2_finish<TT>(a, ob0, lane, acc0, route);
-    fc2_finish<TT>(a, ob0 + 1, lane, acc1, route);
+        for (int tt = 0; tt < TT; ++tt) acc[t][tt] = v4f{0.f, 0.f, 0.f, 0.f};
+    gemm_chunk_lds<TT>(acc, wp, sp, sx, int(ksteps), row, wv, lane, lds);
+    const uint32_t lane2 = after_loop(lane), r2 = lane2 & 15;
+    int32_t route[TT];
+#pragma unroll
+    for (int tt = 0; tt < TT; ++tt) {
+        const bool live = tt < ch.groups && int32_t(r2) < grp[tt].rows;
+        route[tt] = live ? a.plan.original[grp[tt].route_base + r2] : -1;
+    }
+    fc2_finish<TT>(a, ob, lane2, acc, route);
 }
 
-// grid (I/256, chunk capacity), 256 threads. Chunks of one or two groups run the register-only
-// bodies (each wave is independent there, two column blocks in turn); larger chunks share
-// activations through LDS.
-__global__ void __launch_bounds__(kTileThreads) fc1_tile_kernel(Fc1Args a) {
+// Work item of a tile workgroup. Workgroups are handed to the eight XCDs in turn, each with an L2 of
+// its own: the `columns` workgroups of one chunk all take ids of one residue mod 8, so a chunk's
+// activation rows enter one L2 only. The grid is columns * (chunk capacity rounded up to 8).
+struct TileItem { uint32_t chunk, column; };
+__device__ __forceinline__ TileItem tile_item(uint32_t columns) {
+    const uint32_t id = blockIdx.x, xcd = id & 7, slot = id >> 3;
+    return TileItem{(slot / columns) * 8 + xcd, slot % columns};
+}
+__host__ inline uint32_t tile_grid(uint32_t columns, uint32_t chunk_cap) { return columns * ((chunk_cap + 7) / 8 * 8); }
+
+// 256 threads, one workgroup per (chunk, 128 intermediate columns). Chunks of one or two groups run
+// the register-only bodies (each wave is independent there); larger chunks share activations
+// through LDS.
+__global__ void __launch_bounds__(kTileThreads, 2) fc1_tile_kernel(Fc1Args a) {
     extern __shared__ __align__(16) uint8_t lds[];
     uint32_t* meta = a.plan.meta;
-    const uint32_t c = blockIdx.y;
+    const TileItem it = tile_item(a.lay.inter / 128);
+    const uint32_t c = it.chunk;
     if (meta[kPlanFault] || c >= meta[kChunkCount]) return;
     const Chunk ch = a.plan.chunks[c];
-    const uint32_t lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    const uint32_t lane = threadIdx.x & 63, wv = threadIdx.x >> 6, cb = it.column * 4 + wv;
     const int32_t expert = a.plan.groups[ch.first_group].expert;
     if (expert < 0 || expert >= int32_t(kExperts) || ch.groups < 1 || ch.groups > 8) {
         if (lane == 0) atomicOr(&meta[kFc1Fault], 2u);
         return;
     }
-    if (ch.groups <= 2) {
-        for (uint32_t i = 0; i < 2; ++i) {
-            const uint32_t cb = blockIdx.x * 8 + wv * 2 + i;
-            if (ch.groups == 1) fc1_body<1>(a, ch, cb, lane);
-            else fc1_body<2>(a, ch, cb, lane);
-        }
-    } else if (ch.groups <= 4) fc1_tile_body<4>(a, ch, wv, lane, lds);
-    else fc1_tile_body<8>(a, ch, wv, lane, lds);
+    if (ch.groups == 1) fc1_body<1>(a, ch, cb, lane);
+    else if (ch.groups == 2) fc1_body<2>(a, ch, cb, lane);
+    else if (ch.groups <= 4) fc1_tile_body<4>(a, ch, c, cb, wv, lane, lds);
+    else fc1_tile_body<8>(a, ch, c, cb, wv, lane, lds);
 }
 
-// grid (8, chunk capacity), 256 threads: 512 output columns per workgroup.
-__global__ void __launch_bounds__(kTileThreads) fc2_tile_kernel(Fc2Args a) {
+// 256 threads, one workgroup per (chunk, 256 output columns).
+__global__ void __launch_bounds__(kTileThreads, 2) fc2_tile_kernel(Fc2Args a) {
     extern __shared__ __align__(16) uint8_t lds[];
     uint32_t* meta = a.plan.meta;
-    const uint32_t c = blockIdx.y;
+    const TileItem it = tile_item(kHidden / 256);
+    const uint32_t c = it.chunk;
     if (meta[kPlanFault] || meta[kFc1Fault] || meta[kQuantFault] || c >= meta[kChunkCount]) return;
     const Chunk ch = a.plan.chunks[c];
-    const uint32_t lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    const uint32_t lane = threadIdx.x & 63, wv = threadIdx.x >> 6, ob = it.column * 4 + wv;
     const int32_t expert = a.plan.groups[ch.first_group].expert;
     if (expert < 0 || expert >= int32_t(kExperts) || ch.groups < 1 || ch.groups > 8) {
         if (lane == 0) atomicOr(&meta[kFc2Fault], 2u);
         return;
     }
-    if (ch.groups <= 2) {
-        for (uint32_t i = 0; i < 2; ++i) {
-            const uint32_t ob = blockIdx.x * 8 + wv * 2 + i;
-            if (ch.groups == 1) fc2_body<1>(a, ch, ob, lane);
-            else fc2_body<2>(a, ch, ob, lane);
-        }
-    } else if (ch.groups <= 4) fc2_tile_body<4>(a, ch, wv, lane, lds);
-    else fc2_tile_body<8>(a, ch, wv, lane, lds);
+    if (ch.groups == 1) fc2_body<1>(a, ch, ob, lane);
+    else if (ch.groups == 2) fc2_body<2>(a, ch, ob, lane);
+    else if (ch.groups <= 4) fc2_tile_body<4>(a, ch, c, ob, wv, lane, lds);
+    else fc2_tile_body<8>(a, ch, c, ob, wv, lane, lds);
 }
 
 }  // namespace m26g
