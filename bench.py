@@ -193,7 +193,7 @@ def main():
             "workload": "configs[3]: one full MoE layer, prefill chunk, 8192 tokens, Zipf(1.1) routing",
             "value": pw.rows / (pre["ms_per_step"] * 1e-3), "unit": "routed tok/s per MoE layer",
             "ms_per_step": pre["ms_per_step"], "steps": max(3, args.steps // 5),
-            "roofline": {"bound": "mfma", "kernel": "fc1_kernel<8>", "achieved": fc1_tf, "peak": MFMA_FP8_PEAK_TFLOPS,
+            "roofline": {"bound": "mfma", "kernel": "fc1_tile_kernel (gate/up GEMM + SwiGLU + requant)", "achieved": fc1_tf, "peak": MFMA_FP8_PEAK_TFLOPS,
                          "unit": "TFLOP/s", "frac": fc1_tf / MFMA_FP8_PEAK_TFLOPS, "traffic": None,
                          "algorithmic_flops": fc1_flops, "kernel_ms": pre["phases"]["fc1_ms"],
                          "path": {"algorithmic_flops": flops, "achieved": tf, "frac": tf / MFMA_FP8_PEAK_TFLOPS,

@@ -475,6 +475,8 @@ struct Fc1Args {
 // the four lanes that share a row, frexp-rule exponent, exact-grid RNE, reconstruction check), packed
 // stores of payload and scale. `bad` must already be uniform over the four lanes of a row. dg_chunk,
 // when given, also receives the scale byte in the order FC2's tile schedule reads (see Fc1Args::dg).
+// SERIAL computes one activation at a time, for callers whose k-loop registers are still live.
+template <bool SERIAL>
 __device__ __forceinline__ void fc1_finish_tile(const Fc1Args& a, const Chunk ch, uint32_t cb, uint32_t lane, int tt,
                                                 const v4f (&acc)[4], uint32_t bad, bool live, uint8_t* dg_chunk) {
     uint32_t* meta = a.plan.meta;
@@ -488,7 +490,7 @@ __device__ __forceinline__ void fc1_finish_tile(const Fc1Args& a, const Chunk ch
             h[t2][i] = silu_up(acc[t2][i], acc[t2 + 2][i]);
             const uint32_t m = __float_as_uint(h[t2][i]) & 0x7fffffffu;
             amax = m > amax ? m : amax;
-            __builtin_amdgcn_sched_barrier(0);  // one activation at a time: bounds live registers
+            if (SERIAL) __builtin_amdgcn_sched_barrier(0);  // bounds live registers
         }
     uint32_t o = __shfl_xor(amax, 16);
     amax = o > amax ? o : amax;
@@ -545,7 +547,7 @@ __device__ __forceinline__ void fc1_finish(const Fc1Args& a, const Chunk ch, uin
 #pragma unroll
     for (int tt = 0; tt < TT; ++tt) {
         const v4f tile[4] = {acc[0][tt], acc[1][tt], acc[2][tt], acc[3][tt]};
-        fc1_finish_tile(a, ch, cb, lane, tt, tile, bad, live[tt], nullptr);
+        fc1_finish_tile<true>(a, ch, cb, lane, tt, tile, bad, live[tt], nullptr);
     }
 }
 

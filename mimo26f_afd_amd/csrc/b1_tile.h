@@ -174,6 +174,10 @@ __device__ __forceinline__ void gemm_chunk_lds(v4f (&acc)[4][TT], const uint8_t*
     lds_barrier();
     uint32_t wr = 0, ar = 0;  // weight stage that takes step k+2; activation stage of step k
     int q = 0;
+    // The SIMD issues from its oldest wave first, and the other workgroup's wave is usually the older
+    // one, deep in an epilogue of plain vector work: left alone it keeps the issue port and the matrix
+    // pipe idles. Waves in the k-loop therefore outrank everything else.
+    __builtin_amdgcn_s_setprio(3);
     // One k-step with MFMA scale select b = ks % 4 (an immediate, hence the macro).
 #define M26G_KSTEP(b, SW, SA)                                                                                  \
     {                                                                                                          \
@@ -228,6 +232,7 @@ __device__ __forceinline__ void gemm_chunk_lds(v4f (&acc)[4][TT], const uint8_t*
     if (q < quads) M26G_QUAD(sw0, sa0, sw1, sa1)  // odd count: an even number of quads ends on set 0
 #undef M26G_QUAD
 #undef M26G_KSTEP
+    __builtin_amdgcn_s_setprio(0);
     wait_loads_but<0>();  // the re-staged tail loads must land before the LDS is reused or the wave ends
     // The MFMAs above are opaque to the compiler's hazard tracking: let the last ones retire before
     // the epilogue reads the accumulators (8 passes of 4 cycles, plus margin).
@@ -287,7 +292,7 @@ __device__ __forceinline__ void fc1_tile_body(const Fc1Args& a, const Chunk ch, 
         v4f tile[4];
 #pragma unroll
         for (int t = 0; t < 4; ++t) tile[t] = *reinterpret_cast<const v4f*>(bounce + slot + t * 1024);
-        fc1_finish_tile(a, ch, cb, lane2, tt, tile, bad, live[tt], dg_chunk);
+        fc1_finish_tile<false>(a, ch, cb, lane2, tt, tile, bad, live[tt], dg_chunk);
     }
 }
 
@@ -338,6 +343,20 @@ __device__ __forceinline__ TileItem tile_item(uint32_t columns) {
 }
 __host__ inline uint32_t tile_grid(uint32_t columns, uint32_t chunk_cap) { return columns * ((chunk_cap + 7) / 8 * 8); }
 
+// The two workgroups of a compute unit only hide each other's non-MFMA phases when they are out of
+// step, and two that start together stay together (same work, same length). So of the workgroups
+// that start the launch, those in the odd wave slot of their SIMD begin about half a workgroup late;
+// their successors inherit the offset. `naps` counts sleeps of 64*127 cycles.
+#ifndef M26G_NAPS
+#define M26G_NAPS 1
+#endif
+__device__ __forceinline__ void stagger_start(uint32_t naps) {
+    if (!M26G_NAPS || blockIdx.x >= 512) return;
+    const uint32_t wave_slot = __builtin_amdgcn_s_getreg((3 << 11) | (0 << 6) | 4);  // HW_ID bits 3:0
+    if (wave_slot & 1)
+        for (uint32_t i = 0; i < naps; ++i) __builtin_amdgcn_s_sleep(127);
+}
+
 // 256 threads, one workgroup per (chunk, 128 intermediate columns). Chunks of one or two groups run
 // the register-only bodies (each wave is independent there); larger chunks share activations
 // through LDS.
@@ -354,6 +373,7 @@ __global__ void __launch_bounds__(kTileThreads, 2) fc1_tile_kernel(Fc1Args a) {
         if (lane == 0) atomicOr(&meta[kFc1Fault], 2u);
         return;
     }
+    stagger_start(4);
     if (ch.groups == 1) fc1_body<1>(a, ch, cb, lane);
     else if (ch.groups == 2) fc1_body<2>(a, ch, cb, lane);
     else if (ch.groups <= 4) fc1_tile_body<4>(a, ch, c, cb, wv, lane, lds);
@@ -374,6 +394,7 @@ __global__ void __launch_bounds__(kTileThreads, 2) fc2_tile_kernel(Fc2Args a) {
         if (lane == 0) atomicOr(&meta[kFc2Fault], 2u);
         return;
     }
+    stagger_start(3);
     if (ch.groups == 1) fc2_body<1>(a, ch, ob, lane);
     else if (ch.groups == 2) fc2_body<2>(a, ch, ob, lane);
     else if (ch.groups <= 4) fc2_tile_body<4>(a, ch, c, ob, wv, lane, lds);
