@@ -274,34 +274,18 @@ __device__ __forceinline__ int quant_scale_exponent(uint32_t amax_bits) {
     return int(a >> 23) - 127 - ((a & 0x7fffffu) <= 0x600000u ? 8 : 7);
 }
 
-// Round-half-even of value / 2^shift for value < 2^24, shift >= 1.
-__device__ __forceinline__ uint32_t rne_shift(uint32_t value, int shift) {
-    if (shift > 25) return 0;
-    const uint32_t q = value >> shift, rem = value & ((1u << shift) - 1u), half = 1u << (shift - 1);
-    return q + ((rem > half || (rem == half && (q & 1u))) ? 1u : 0u);
+// E4M3FN codes of h0 * 2^-k and h1 * 2^-k in the two low bytes (h0 lowest), on top of `old`'s other
+// half when HIGH. The scaling is exact (a power of two; where it would underflow the product is far
+// below half the E4M3 quantum anyway) and gfx950's conversion is the OCP one: round to nearest even,
+// subnormals kept, sign of zero kept. |h| <= amax <= 448 * 2^k, so nothing saturates.
+template <bool HIGH>
+__device__ __forceinline__ uint32_t quant_pair(float h0, float h1, int k, uint32_t old = 0) {
+    return uint32_t(__builtin_amdgcn_cvt_pk_fp8_f32(__builtin_ldexpf(h0, -k), __builtin_ldexpf(h1, -k), int(old), HIGH));
 }
+__device__ __forceinline__ uint32_t quant_code(float h, int k) { return quant_pair<false>(h, 0.0f, k) & 0xffu; }
 
-// E4M3FN code of h * 2^-k, ties to even, sign of zero kept.
-__device__ __forceinline__ uint32_t quant_code(uint32_t bits, int k) {
-    const uint32_t sign = (bits >> 24) & 0x80u, mag = bits & 0x7fffffffu;
-    if (!mag) return sign;
-    const uint32_t field = mag >> 23;
-    // A subnormal input is far below the floor-derived quantum: it rounds to zero for every legal k.
-    if (!field) return sign;
-    const uint32_t sig = (mag & 0x7fffffu) | 0x800000u;
-    int e = int(field) - 127 - k;
-    uint32_t code;
-    if (e < -6) {
-        code = rne_shift(sig, 14 - e);  // quantum 2^-9; a carry into 8 is the first normal code
-    } else {
-        uint32_t r = rne_shift(sig, 20);
-        if (r == 16) { r = 8; ++e; }
-        code = uint32_t(e + 7) * 8 + r - 8;
-        if (code > 126) code = 126;
-    }
-    return sign | code;
-}
-
+// The reconstruction code * 2^k leaves FP32 only for a normal code with field - 7 + k > 127, which
+// needs k >= 120: blocks below that skip the check.
 __device__ __forceinline__ bool quant_reconstructs(uint32_t code, int k) {
     const uint32_t field = (code & 0x7fu) >> 3;
     return field == 0 || int(field) - 7 + k <= 127;
@@ -327,7 +311,7 @@ __global__ void __launch_bounds__(256) quantize_kernel(const float* __restrict__
             continue;
         }
         const int k = quant_scale_exponent(amax);
-        const uint32_t code = quant_code(bits, k);
+        const uint32_t code = quant_code(__uint_as_float(bits), k);
         uint32_t over = quant_reconstructs(code, k) ? 0u : 1u;
 #pragma unroll
         for (int d = 16; d; d >>= 1) over |= __shfl_xor(over, d);
@@ -413,39 +397,28 @@ __device__ __forceinline__ void gemm_chunk(v4f (&acc)[4][TT], const uint8_t* __r
     }
 }
 
-// e^t for t <= 0 as the CPU reference forms it: evaluated in binary64, rounded once to binary32
-// (mimo26-repack/tests/lattice_oracle.py:32-53 uses libm's binary64 exp). Cody-Waite reduction by
-// ln 2 and an 11th-degree Taylor polynomial on |r| <= 0.347 keep the binary64 value within a few
-// ulp (2^-47 truncation), so the binary32 rounding differs from libm's only when the exact value
-// lies within ~1e-15 of a rounding boundary. About twenty FP64 operations, few live registers.
-__device__ __forceinline__ float exp_nonpositive(float tf) {
-    const double t = double(tf);
-    const double n = __builtin_rint(t * 1.4426950408889634074);
-    double r = __builtin_fma(n, -6.93147180369123816490e-01, t);
-    r = __builtin_fma(n, -1.90821492927058770002e-10, r);
-    double p = 2.50521083854417187751e-08;  // 1/11!
-    p = __builtin_fma(p, r, 2.75573192239858906526e-07);
-    p = __builtin_fma(p, r, 2.75573192239858906526e-06);
-    p = __builtin_fma(p, r, 2.48015873015873015873e-05);
-    p = __builtin_fma(p, r, 1.98412698412698412698e-04);
-    p = __builtin_fma(p, r, 1.38888888888888888889e-03);
-    p = __builtin_fma(p, r, 8.33333333333333333333e-03);
-    p = __builtin_fma(p, r, 4.16666666666666666667e-02);
-    p = __builtin_fma(p, r, 1.66666666666666666667e-01);
-    p = __builtin_fma(p, r, 0.5);
-    p = __builtin_fma(p, r, 1.0);
-    p = __builtin_fma(p, r, 1.0);
-    return float(__builtin_ldexp(p, int(n)));
+// e^t for t <= 0 in binary32: Cody-Waite reduction by ln 2 (two FMAs), the hardware 2^x on the
+// remainder, exponent put back with ldexp. Within 2 ulp of the true value, the accuracy class of the
+// expf the reference's own kernels call (crates/mimo26-expert/kernels/b1/grouped.cu:89).
+__device__ __forceinline__ float exp_nonpositive(float t) {
+    const float n = __builtin_rintf(t * 1.44269504088896340736f);
+    float r = __builtin_fmaf(n, -0.693145751953125f, t);
+    r = __builtin_fmaf(n, -1.42860682030941723212e-06f, r);
+    return __builtin_ldexpf(__builtin_amdgcn_exp2f(r * 1.44269504088896340736f), int(n));
 }
 
 // SwiGLU in the reference's stable form (kernels/b1/grouped.cu:89-93): e = exp(-|g|);
-// s = g >= 0 ? g/(1+e) : (g*e)/(1+e); h = s*u, every step one FP32 rounding.
+// s = g >= 0 ? g/(1+e) : (g*e)/(1+e); h = s*u. The quotient is a reciprocal plus one Newton step on
+// the residual (within 1 ulp). The whole activation stays within a few binary32 ulp of the CPU rule,
+// which rounds every step once; the epilogues are bound by vector-instruction issue, and the exactly
+// rounded form costs three times the instructions.
 __device__ __forceinline__ float silu_up(float g, float u) {
-    const float t = g >= 0.0f ? -g : g;
-    const float e = exp_nonpositive(t);
-    const float d = __fadd_rn(1.0f, e);
-    const float s = g >= 0.0f ? __fdiv_rn(g, d) : __fdiv_rn(__fmul_rn(g, e), d);
-    return __fmul_rn(s, u);
+    const float e = exp_nonpositive(g >= 0.0f ? -g : g);
+    const float d = 1.0f + e, num = g >= 0.0f ? g : g * e;
+    const float rc = __builtin_amdgcn_rcpf(d);
+    float q = num * rc;
+    q = __builtin_fmaf(__builtin_fmaf(-d, q, num), rc, q);
+    return q * u;
 }
 
 struct Fc1Args {
@@ -509,18 +482,21 @@ __device__ __forceinline__ void fc1_finish_tile(const Fc1Args& a, const Chunk ch
     const uint32_t block = uint32_t(grow * (I / 32) + cb);
     uint32_t fault = (amax >= 0x7f800000u || bad) ? 1u : 0u;
     const int k = quant_scale_exponent(amax);
-    uint32_t word[2] = {0, 0};
+    uint32_t word[2];
     uint32_t over = 0;
 #pragma unroll
-    for (int t2 = 0; t2 < 2; ++t2)
+    for (int t2 = 0; t2 < 2; ++t2) {
+        word[t2] = quant_pair<false>(h[t2][0], h[t2][1], k);
+        word[t2] = quant_pair<true>(h[t2][2], h[t2][3], k, word[t2]);
+    }
+    if (__ballot(k >= 120)) {  // wave-uniform, and practically never taken
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const uint32_t code = quant_code(__float_as_uint(h[t2][i]), k);
-            over |= quant_reconstructs(code, k) ? 0u : 1u;
-            word[t2] |= code << (8 * i);
-        }
-    over |= __shfl_xor(over, 16);
-    over |= __shfl_xor(over, 32);
+        for (int t2 = 0; t2 < 2; ++t2)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) over |= quant_reconstructs((word[t2] >> (8 * i)) & 0xffu, k) ? 0u : 1u;
+        over |= __shfl_xor(over, 16);
+        over |= __shfl_xor(over, 32);
+    }
     if (!fault && over) fault = 2;
     if (!live) return;
     if (fault) {

@@ -274,25 +274,35 @@ __device__ __forceinline__ void fc1_tile_body(const Fc1Args& a, const Chunk ch, 
     gemm_chunk_lds<TT>(acc, wp, sp, sx, int(kHidden / 128), row, wv, lane, lds);
     const uint32_t lane2 = after_loop(lane), r2 = lane2 & 15;
     const uint32_t bad = a.rowbad[c * 16 + r2];
-    bool live[TT];
-#pragma unroll
-    for (int tt = 0; tt < TT; ++tt) live[tt] = tt < ch.groups && grp[tt].input_rows[r2] >= 0;
-    // The accumulators leave the accumulation registers through the wave's own, now idle, weight ring:
-    // whole-tile LDS writes keep them out of the register allocator's hands until the very end (element
-    // reads straight from the accumulation file make it split their live ranges across the k-loop).
-    uint8_t* bounce = lds + wv * (kWeightStages * 4096) + lane2 * 16;
+    // The accumulators leave the accumulation registers through LDS, sixteen tiles at a time: whole-tile
+    // writes keep them out of the register allocator's hands until the very end (element reads straight
+    // from the accumulation file make it split their live ranges across the k-loop), and the epilogue
+    // becomes one rolled loop over the activation tiles. Unrolled it is 70 KB of code, and two workgroups
+    // in different phases then evict each other's instructions from the cache the compute units share.
+    // Every wave has drained its own direct loads; after the barrier nobody's are left, and each wave
+    // takes a quarter of the first 64 KB.
+    asm volatile("s_barrier" ::: "memory");
+    uint8_t* bounce = lds + wv * 16384 + lane2 * 16;
     const uint32_t bounce_at = uint32_t(uintptr_t((lds_ptr)bounce));
+    auto park = [&](int half) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+                asm volatile("ds_write_b128 %0, %1 offset:%2" ::"v"(bounce_at), "a"(acc[t][(TT == 8 ? half * 4 : 0) + j]),
+                             "n"((j * 4 + t) * 1024)
+                             : "memory");
+    };
     uint8_t* dg_chunk = a.dg + size_t(c) * gathered_scale_bytes(a.lay.inter);
-#pragma unroll
+    park(0);
+#pragma unroll 1
     for (int tt = 0; tt < TT; ++tt) {
-        const uint32_t slot = (tt & 1) * 4096;
-#pragma unroll
-        for (int t = 0; t < 4; ++t)
-            asm volatile("ds_write_b128 %0, %1" ::"v"(bounce_at + slot + t * 1024), "a"(acc[t][tt]) : "memory");
+        if (TT == 8 && tt == 4) park(1);  // in-order LDS: the first half has been read by now
         v4f tile[4];
 #pragma unroll
-        for (int t = 0; t < 4; ++t) tile[t] = *reinterpret_cast<const v4f*>(bounce + slot + t * 1024);
-        fc1_finish_tile<false>(a, ch, cb, lane2, tt, tile, bad, live[tt], dg_chunk);
+        for (int t = 0; t < 4; ++t) tile[t] = *reinterpret_cast<const v4f*>(bounce + ((tt & 3) * 4 + t) * 1024);
+        const bool live = tt < ch.groups && grp[tt < ch.groups ? tt : 0].input_rows[r2] >= 0;
+        fc1_finish_tile<false>(a, ch, cb, lane2, tt, tile, bad, live, dg_chunk);
     }
 }
 

@@ -17,6 +17,7 @@ pytestmark = pytest.mark.gpu
 MAX_ABS, MEAN_REL = 1e-2, 1e-3
 # FP32 accumulation bound for one output: one rounding per 128-wide k-step plus the MFMA's internal
 # sum, against the FP64 ideal: a small multiple of 2^-24 times the sum of |products|.
+SILU_ULPS = 8.0
 ACC_EPS = 8 * 2.0 ** -24
 
 
@@ -56,7 +57,11 @@ def check_stages(scratch, layer, wl, pools, stats, experts=3):
             assert np.max(err) <= ACC_EPS * 4096 * np.max(x) * 6 * 2.0 ** -4, (k, np.max(err))
             assert parity(taps[k][sl], want[k])[1] < 1e-5
         assert parity(taps["h"][sl], want["h"])[1] < 1e-4
-        assert np.array_equal(taps["h"][sl], O.silu_up(taps["gate"][sl], taps["up"][sl]))       # activation bit-exact on its inputs
+        # The activation on its own inputs: the CPU rule rounds every step once, the kernel uses the
+        # hardware 2^x and a refined reciprocal (the reference's kernels call expf): a few binary32 ulp.
+        rule = O.silu_up(taps["gate"][sl], taps["up"][sl])
+        ulps = np.abs(taps["h"][sl].astype(np.float64) - rule) / np.spacing(np.maximum(np.abs(rule), np.float32(2.0 ** -100)))
+        assert np.max(ulps) <= SILU_ULPS, np.max(ulps)
         qp, qs, qf = O.quant_v1(taps["h"][sl])
         assert not qf.any() and np.array_equal(qp, mp[sl]) and np.array_equal(qs, ms[sl])       # codec bytes on the reported h
         assert np.mean(mp[sl] == want["mid_payload"]) > 0.995
