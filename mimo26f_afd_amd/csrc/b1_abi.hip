@@ -212,7 +212,7 @@ int enqueue(const m26s_b1_layer* L, m26s_b1_scratch* S, const uint8_t* x, size_t
                       S->chunks.as<Chunk>(), S->meta.as<uint32_t>()};
     M26S_CK(hipEventRecord(S->e0, S->st), "b1 event 0");
     // Stage faults accumulate across enqueued calls until the next sync; only the plan words reset.
-    plan_kernel<<<1, kPlanThreads, routes, S->st>>>(ids, w, rows, L->resident, pv, nt, 0);
+    plan_kernel<<<1, kPlanThreads, routes, S->st>>>(ids, w, rows, L->resident, pv, nt, 0, S->taps);
     M26S_CK(hipGetLastError(), "b1 plan launch");
     M26S_CK(hipEventRecord(S->ep, S->st), "b1 event p");
     if (nt == 1) launch_ffn<1>(L, S, pv, x, xp, xs, xsp, uint32_t(ccap), routes);
@@ -416,7 +416,7 @@ int m26s_b1_plan_dev(const int32_t* ids_dev, const float* weights_dev, uint32_t 
                       chunks.as<Chunk>(), meta.as<uint32_t>()};
     uint32_t m[kMetaWords];
     plan_kernel<<<1, kPlanThreads, uint64_t(rows) * kTopk, 0>>>(ids_dev, weights_dev, rows, resident_dev, pv, 1,
-                                                                 capacity * kTopk);
+                                                                 capacity * kTopk, true);
     M26S_CK(hipGetLastError(), "b1 plan launch");
     M26S_CK(hipMemcpy(m, meta.p, sizeof m, hipMemcpyDeviceToHost), "b1 plan meta download");
     M26S_CK(hipMemcpy(fault_dev, &m[kPlanFault], 4, hipMemcpyHostToDevice), "b1 plan fault store");

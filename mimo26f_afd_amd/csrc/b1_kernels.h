@@ -138,11 +138,12 @@ __device__ __forceinline__ uint32_t last_not_above(const uint32_t* base, uint32_
 
 __global__ void __launch_bounds__(kPlanThreads)
 plan_kernel(const int32_t* __restrict__ ids, const float* __restrict__ w, uint32_t rows,
-            const uint8_t* __restrict__ resident, PlanView p, uint32_t gpc, uint32_t reset_capacity) {
-    extern __shared__ uint8_t id_byte[];
+            const uint8_t* __restrict__ resident, PlanView p, uint32_t gpc, uint32_t reset_capacity, bool want_gw) {
+    extern __shared__ __align__(16) uint8_t id_byte[];
     __shared__ uint32_t hist[kPlanWaves][256];
     __shared__ uint32_t cnt[256], rbase[257], gbase[257], cbase[257];
     __shared__ uint32_t first_bad;
+    __shared__ uint8_t present[256];
     const uint32_t tid = threadIdx.x, lane = tid & 63, wv = tid >> 6, routes = rows * kTopk;
 
     for (uint32_t i = tid; i < kPlanWaves * 256; i += kPlanThreads) (&hist[0][0])[i] = 0;
@@ -150,15 +151,42 @@ plan_kernel(const int32_t* __restrict__ ids, const float* __restrict__ w, uint32
     __syncthreads();
     // Validation keys order faults as the serial planner meets them: (route + 1) << 4 | check,
     // check 1 = id or residency, 2 = weight, 3 = expert repeated inside the token.
-    if (tid < 256 && resident[tid] > 1) atomicMin(&first_bad, 1u);
-    for (uint32_t i = tid; i < routes; i += kPlanThreads) {
-        const int32_t e = ids[i];
-        const float wt = w[i];
-        uint32_t check = 0;
-        if (e < 0 || e >= int32_t(kExperts) || !resident[e]) check = 1;
-        else if (!(wt >= 0.0f && wt <= FLT_MAX)) check = 2;
-        if (check) atomicMin(&first_bad, ((i + 1) << 4) | check);
-        id_byte[i] = uint8_t(e);
+    if (tid < 256) {
+        const uint8_t here = resident[tid];
+        if (here > 1) atomicMin(&first_bad, 1u);
+        present[tid] = here;
+    }
+    __syncthreads();
+    // One token (its eight routes) per thread and trip, two trips in flight: the walk is bound by the
+    // latency of these loads, not by their volume.
+    auto check_token = [&](uint32_t t, const v4i& ia, const v4i& ib, const v4f& wa, const v4f& wb) {
+        const int32_t e8[8] = {ia.x, ia.y, ia.z, ia.w, ib.x, ib.y, ib.z, ib.w};
+        const float w8[8] = {wa.x, wa.y, wa.z, wa.w, wb.x, wb.y, wb.z, wb.w};
+        uint32_t packed[2] = {0, 0};
+#pragma unroll
+        for (uint32_t j = 0; j < 8; ++j) {
+            const int32_t e = e8[j];
+            uint32_t check = 0;
+            if (e < 0 || e >= int32_t(kExperts) || !present[e & 255]) check = 1;
+            else if (!(w8[j] >= 0.0f && w8[j] <= FLT_MAX)) check = 2;
+            if (check) atomicMin(&first_bad, ((t * 8 + j + 1) << 4) | check);
+            packed[j >> 2] |= (uint32_t(e) & 0xffu) << (8 * (j & 3));
+        }
+        *reinterpret_cast<uint2*>(id_byte + t * 8) = uint2{packed[0], packed[1]};
+    };
+    typedef v4i __attribute__((aligned(4))) v4i_u;
+    typedef v4f __attribute__((aligned(4))) v4f_u;
+    const v4i_u* ids4 = reinterpret_cast<const v4i_u*>(ids);
+    const v4f_u* w4 = reinterpret_cast<const v4f_u*>(w);
+    for (uint32_t t = tid; t < rows; t += 2 * kPlanThreads) {
+        const uint32_t u = t + kPlanThreads;
+        const bool two = u < rows;
+        const v4i ia = ids4[2 * t], ib = ids4[2 * t + 1];
+        const v4f wa = w4[2 * t], wb = w4[2 * t + 1];
+        const v4i ic = ids4[two ? 2 * u : 2 * t], id = ids4[two ? 2 * u + 1 : 2 * t + 1];
+        const v4f wc = w4[two ? 2 * u : 2 * t], wd = w4[two ? 2 * u + 1 : 2 * t + 1];
+        check_token(t, ia, ib, wa, wb);
+        if (two) check_token(u, ic, id, wc, wd);
     }
     __syncthreads();
     const uint32_t run = (((routes + kPlanWaves - 1) / kPlanWaves) + 63u) & ~63u;
@@ -234,7 +262,22 @@ plan_kernel(const int32_t* __restrict__ ids, const float* __restrict__ w, uint32
         }
     }
     __syncthreads();
-    for (uint32_t i = tid; i < routes; i += kPlanThreads) p.gw[p.inverse[i]] = w[i];
+    // Weights in grouped order: part of the planner's output, but nothing downstream reads it (the
+    // combine takes the caller's weights by route), so the FFN path only fills it for the taps.
+    if (want_gw)
+        for (uint32_t s0 = tid; s0 < routes; s0 += 8 * kPlanThreads) {
+            float wt[8];
+            int32_t at[8];
+#pragma unroll
+            for (uint32_t j = 0; j < 8; ++j) {
+                const uint32_t i = s0 + j * kPlanThreads;
+                wt[j] = i < routes ? w[i] : 0.0f;
+                at[j] = i < routes ? p.inverse[i] : -1;
+            }
+#pragma unroll
+            for (uint32_t j = 0; j < 8; ++j)
+                if (at[j] >= 0) p.gw[at[j]] = wt[j];
+        }
     const uint32_t ngroups = gbase[256], nchunks = cbase[256];
     for (uint32_t gi = tid; gi < ngroups; gi += kPlanThreads) {
         const uint32_t e = last_not_above(gbase, gi), k = gi - gbase[e];
@@ -439,7 +482,8 @@ struct Fc1Args {
     // Tile schedule only: per-chunk activation scales in MFMA lane order, [chunk][K/512][8 tiles][64 lanes]
     // dwords whose byte b is the scale of k-block 4*(4q+b) + lane/16 of row lane%16.
     const uint8_t* xg;     // FC1 input scales, gathered by gather_scales_kernel
-    const uint32_t* rowbad;  // [chunk][16]: nonzero where a row index of the chunk met an illegal input scale
+    const uint32_t* rowbad;  // [chunk][16]: bit 0 set where a row index of the chunk met an illegal input scale,
+                             // bit 8+t set where tile t holds a token in that row
     uint8_t* dg;           // the intermediate's scales in the same order, written here for FC2
 };
 

@@ -71,8 +71,9 @@ __device__ __forceinline__ void mfma_acc(v4f& acc, const v4i& a, const v8i& b, u
 
 // Rewrites the activation scale rows of every chunk into MFMA lane order (layout at Fc1Args::xg) and
 // checks them against the legal window [105, 247] (crates/mimo26-expert/kernels/b1/grouped.cu:28,37
-// holds the reference's check). Padded rows get the unit scale 127. rowbad[chunk][r] collects the
-// verdict of row r of all tiles, the granularity the FC1 epilogue reports faults at.
+// holds the reference's check). Padded rows get the unit scale 127. rowbad[chunk][r] collects, for
+// row r of all tiles, the verdict in bit 0 (the granularity the FC1 epilogue reports faults at) and
+// in bit 8+t whether tile t holds a token there, so the epilogue looks nothing else up.
 // grid (chunk capacity), 256 threads = 8 tiles x 16 rows x 2 halves of a scale row.
 __global__ void __launch_bounds__(256) gather_scales_kernel(PlanView plan, const uint8_t* __restrict__ xs, size_t xs_pitch,
                                                             uint32_t* __restrict__ xg, uint32_t* __restrict__ rowbad) {
@@ -109,7 +110,8 @@ __global__ void __launch_bounds__(256) gather_scales_kernel(PlanView plan, const
             xg[((size_t(c) * (kHidden / 512) + q) * 8 + tt) * 64 + g * 16 + r] = out;
         }
     }
-    if (bad) atomicOr(&flags[r], 1u);
+    const uint32_t verdict = bad | (row >= 0 ? 0x100u << tt : 0u);
+    if (verdict) atomicOr(&flags[r], verdict);
     __syncthreads();
     if (tid < 16) rowbad[c * 16 + tid] = flags[tid];
 }
@@ -273,7 +275,7 @@ __device__ __forceinline__ void fc1_tile_body(const Fc1Args& a, const Chunk ch, 
         for (int tt = 0; tt < TT; ++tt) acc[t][tt] = v4f{0.f, 0.f, 0.f, 0.f};
     gemm_chunk_lds<TT>(acc, wp, sp, sx, int(kHidden / 128), row, wv, lane, lds);
     const uint32_t lane2 = after_loop(lane), r2 = lane2 & 15;
-    const uint32_t bad = a.rowbad[c * 16 + r2];
+    const uint32_t verdict = a.rowbad[c * 16 + r2], bad = verdict & 1u;
     // The accumulators leave the accumulation registers through LDS, sixteen tiles at a time: whole-tile
     // writes keep them out of the register allocator's hands until the very end (element reads straight
     // from the accumulation file make it split their live ranges across the k-loop), and the epilogue
@@ -301,7 +303,7 @@ __device__ __forceinline__ void fc1_tile_body(const Fc1Args& a, const Chunk ch, 
         v4f tile[4];
 #pragma unroll
         for (int t = 0; t < 4; ++t) tile[t] = *reinterpret_cast<const v4f*>(bounce + ((tt & 3) * 4 + t) * 1024);
-        const bool live = tt < ch.groups && grp[tt < ch.groups ? tt : 0].input_rows[r2] >= 0;
+        const bool live = (verdict >> (8 + tt)) & 1u;
         fc1_finish_tile<false>(a, ch, cb, lane2, tt, tile, bad, live, dg_chunk);
     }
 }
