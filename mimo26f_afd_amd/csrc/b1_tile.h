@@ -50,6 +50,14 @@ template <int N> __device__ __forceinline__ void wait_loads_but() {
     static_assert(N >= 0 && N < 64, "vmcnt immediate");
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
 }
+template <int N> __device__ __forceinline__ void wait_lds_but() {
+    asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(N) : "memory");
+}
+// One lane's 32 bytes of an activation fragment: the two 16-byte cells at `at` and `at` + 1024.
+__device__ __forceinline__ void read_fragment(v4i& lo, v4i& hi, uint32_t at) {
+    asm volatile("ds_read_b128 %0, %1" : "=v"(lo) : "v"(at) : "memory");
+    asm volatile("ds_read_b128 %0, %1 offset:1024" : "=v"(hi) : "v"(at) : "memory");
+}
 // LDS-only workgroup barrier: outstanding global prefetches stay in flight across it.
 __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
@@ -146,10 +154,17 @@ __device__ __forceinline__ void gemm_chunk_lds(v4f (&acc)[4][TT], const uint8_t*
 #pragma unroll
         for (int item = 0; item < kPerStep; ++item) stage_item(item, ks, astage, wstage);
     };
+    // LDS reads are issued by hand too, with their own lgkmcnt waits. Left to the compiler, every wait
+    // on an LDS read is a wait for all of them (it knows of the direct loads above and drains
+    // everything to be safe), the fragment fetched for the next MFMA group included. As with the
+    // scales, nothing but the MFMAs, behind those waits, may read the registers so filled.
+    const uint32_t wring_at = uint32_t(uintptr_t((lds_ptr)wring)) + lane * 16;
+    const uint32_t aring_at = uint32_t(uintptr_t((lds_ptr)aring)) + lane * 16;
     v4i af[2][4];  // weight fragments of this k-step and the next
     auto read_weights = [&](v4i (&a)[4], uint32_t stage) {
+        const uint32_t at = wring_at + stage * 4096;
 #pragma unroll
-        for (int t = 0; t < 4; ++t) a[t] = *reinterpret_cast<const v4i*>(wring + stage * 4096 + t * 1024 + lane * 16);
+        for (int t = 0; t < 4; ++t) asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(a[t]) : "v"(at), "n"(t * 1024) : "memory");
     };
     // Scale dwords of a quad of k-steps (four weight tiles, TT activation tiles), in two register sets
     // that alternate. They are loaded by hand a whole quad ahead: a load the compiler knows of makes
@@ -174,13 +189,18 @@ __device__ __forceinline__ void gemm_chunk_lds(v4f (&acc)[4][TT], const uint8_t*
     wait_loads_but<kPerStep>();  // step 0 and the first scales have landed, step 1 may still fly
     read_weights(af[0], 0);
     lds_barrier();
+    v4i flo, fhi;  // the fragment a k-step starts with
+    read_fragment(flo, fhi, aring_at);
     uint32_t wr = 0, ar = 0;  // weight stage that takes step k+2; activation stage of step k
     int q = 0;
-    // The SIMD issues from its oldest wave first, and the other workgroup's wave is usually the older
-    // one, deep in an epilogue of plain vector work: left alone it keeps the issue port and the matrix
-    // pipe idles. Waves in the k-loop therefore outrank everything else.
-    __builtin_amdgcn_s_setprio(3);
     // One k-step with MFMA scale select b = ks % 4 (an immediate, hence the macro).
+    //
+    // A wave issues in order, roughly one instruction every four or five cycles, while an MFMA holds the
+    // matrix pipe for 32: whatever else the step needs (fragment reads, direct loads with their address
+    // arithmetic) is slotted between the MFMAs of a group, a few instructions per gap, so the pipe never
+    // waits for them. The workgroup barrier sits ahead of the last group's MFMAs, not behind them: what
+    // it orders (every wave's loads of step k+1 landed, every wave's reads of step k done) is true by
+    // then, and the first fragment of step k+1 and the next weights are fetched under those MFMAs.
 #define M26G_KSTEP(b, SW, SA)                                                                                  \
     {                                                                                                          \
         const int ks = 4 * q + (b);                                                                            \
@@ -189,31 +209,47 @@ __device__ __forceinline__ void gemm_chunk_lds(v4f (&acc)[4][TT], const uint8_t*
         const uint32_t ar1 = ar == kActStages - 1 ? 0 : ar + 1, ar2 = ar1 == kActStages - 1 ? 0 : ar1 + 1;     \
         /* Past the end the last step is staged again into stages nobody reads any more. */                   \
         const int ahead = ks + 2 < last ? ks + 2 : last;                                                       \
-        const uint8_t* fs = aring + ar * TT * 2048 + lane * 16;                                                \
-        v4i lo = *reinterpret_cast<const v4i*>(fs), hi = *reinterpret_cast<const v4i*>(fs + 1024);             \
-        __builtin_amdgcn_sched_barrier(0);                                                                     \
+        const uint32_t fs = aring_at + ar * TT * 2048;                                                         \
+        v4i lo = flo, hi = fhi; /* fragment 0, fetched at the end of the step before */                       \
         _Pragma("unroll") for (int tt = 0; tt < TT; ++tt) {                                                    \
-            _Pragma("unroll") for (int item = 0; item < kPerStep; ++item)                                      \
-                if (item * TT / kPerStep == tt) stage_item(item, ahead, ar2, wr);                              \
-            const v8i bv = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};                                   \
-            if (tt + 1 < TT) { /* the next fragment is on its way while this one multiplies */                 \
-                lo = *reinterpret_cast<const v4i*>(fs + (tt + 1) * 2048);                                      \
-                hi = *reinterpret_cast<const v4i*>(fs + (tt + 1) * 2048 + 1024);                               \
-            } else {                                                                                           \
+            v4i nlo = lo, nhi = hi;                                                                            \
+            if (tt == TT - 1) {                                                                                \
+                _Pragma("unroll") for (int item = 0; item < kPerStep; ++item)                                  \
+                    if (item * TT / kPerStep == tt) stage_item(item, ahead, ar2, wr);                          \
+                __builtin_amdgcn_sched_barrier(0);                                                             \
                 /* Everything but this step's own loads (step k+2) has landed: activations and weights */      \
                 /* of step k+1, issued one whole k-step ago, and the next quad's scales, older still.   */      \
                 wait_loads_but<kPerStep>();                                                                    \
+                lds_barrier(); /* with the wait for this group's fragment */                                   \
+                read_fragment(flo, fhi, aring_at + ar1 * TT * 2048);                                           \
                 read_weights(af[((b) + 1) & 1], wr ^ 1);                                                       \
+            } else {                                                                                           \
+                wait_lds_but<0>();                                                                             \
             }                                                                                                  \
             __builtin_amdgcn_sched_barrier(0);                                                                 \
-            _Pragma("unroll") for (int t = 0; t < 4; ++t)                                                      \
-                mfma_acc<(b)>(acc[t][tt], af[(b) & 1][t], bv, SW[t], SA[tt]);                                   \
+            const v8i bv = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};                                   \
+            mfma_acc<(b)>(acc[0][tt], af[(b) & 1][0], bv, SW[0], SA[tt]);                                       \
             __builtin_amdgcn_sched_barrier(0);                                                                 \
+            if (tt + 1 < TT) asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(nlo) : "v"(fs), "n"((tt + 1 < TT ? tt + 1 : 0) * 2048) : "memory"); \
+            __builtin_amdgcn_sched_barrier(0);                                                                 \
+            mfma_acc<(b)>(acc[1][tt], af[(b) & 1][1], bv, SW[1], SA[tt]);                                       \
+            __builtin_amdgcn_sched_barrier(0);                                                                 \
+            if (tt + 1 < TT) asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(nhi) : "v"(fs), "n"((tt + 1 < TT ? tt + 1 : 0) * 2048 + 1024) : "memory"); \
+            __builtin_amdgcn_sched_barrier(0);                                                                 \
+            mfma_acc<(b)>(acc[2][tt], af[(b) & 1][2], bv, SW[2], SA[tt]);                                       \
+            __builtin_amdgcn_sched_barrier(0);                                                                 \
+            if (tt + 1 < TT) {                                                                                 \
+                _Pragma("unroll") for (int item = 0; item < kPerStep; ++item)                                  \
+                    if (item * TT / kPerStep == tt) stage_item(item, ahead, ar2, wr);                          \
+            }                                                                                                  \
+            __builtin_amdgcn_sched_barrier(0);                                                                 \
+            mfma_acc<(b)>(acc[3][tt], af[(b) & 1][3], bv, SW[3], SA[tt]);                                       \
+            __builtin_amdgcn_sched_barrier(0);                                                                 \
+            lo = nlo;                                                                                          \
+            hi = nhi;                                                                                          \
         }                                                                                                      \
         wr ^= 1;                                                                                               \
         ar = ar1;                                                                                              \
-        lds_barrier();                                                                                         \
-        __builtin_amdgcn_sched_barrier(0);                                                                     \
     }
     // A quad: fetch the next quad's scales into the other set, then four k-steps on this set.
 #define M26G_QUAD(SW, SA, NW, NA)                                                                              \
@@ -234,7 +270,6 @@ __device__ __forceinline__ void gemm_chunk_lds(v4f (&acc)[4][TT], const uint8_t*
     if (q < quads) M26G_QUAD(sw0, sa0, sw1, sa1)  // odd count: an even number of quads ends on set 0
 #undef M26G_QUAD
 #undef M26G_KSTEP
-    __builtin_amdgcn_s_setprio(0);
     wait_loads_but<0>();  // the re-staged tail loads must land before the LDS is reused or the wave ends
     // The MFMAs above are opaque to the compiler's hazard tracking: let the last ones retire before
     // the epilogue reads the accumulators (8 passes of 4 cycles, plus margin).
@@ -355,20 +390,6 @@ __device__ __forceinline__ TileItem tile_item(uint32_t columns) {
 }
 __host__ inline uint32_t tile_grid(uint32_t columns, uint32_t chunk_cap) { return columns * ((chunk_cap + 7) / 8 * 8); }
 
-// The two workgroups of a compute unit only hide each other's non-MFMA phases when they are out of
-// step, and two that start together stay together (same work, same length). So of the workgroups
-// that start the launch, those in the odd wave slot of their SIMD begin about half a workgroup late;
-// their successors inherit the offset. `naps` counts sleeps of 64*127 cycles.
-#ifndef M26G_NAPS
-#define M26G_NAPS 1
-#endif
-__device__ __forceinline__ void stagger_start(uint32_t naps) {
-    if (!M26G_NAPS || blockIdx.x >= 512) return;
-    const uint32_t wave_slot = __builtin_amdgcn_s_getreg((3 << 11) | (0 << 6) | 4);  // HW_ID bits 3:0
-    if (wave_slot & 1)
-        for (uint32_t i = 0; i < naps; ++i) __builtin_amdgcn_s_sleep(127);
-}
-
 // 256 threads, one workgroup per (chunk, 128 intermediate columns). Chunks of one or two groups run
 // the register-only bodies (each wave is independent there); larger chunks share activations
 // through LDS.
@@ -385,7 +406,6 @@ __global__ void __launch_bounds__(kTileThreads, 2) fc1_tile_kernel(Fc1Args a) {
         if (lane == 0) atomicOr(&meta[kFc1Fault], 2u);
         return;
     }
-    stagger_start(4);
     if (ch.groups == 1) fc1_body<1>(a, ch, cb, lane);
     else if (ch.groups == 2) fc1_body<2>(a, ch, cb, lane);
     else if (ch.groups <= 4) fc1_tile_body<4>(a, ch, c, cb, wv, lane, lds);
@@ -406,7 +426,6 @@ __global__ void __launch_bounds__(kTileThreads, 2) fc2_tile_kernel(Fc2Args a) {
         if (lane == 0) atomicOr(&meta[kFc2Fault], 2u);
         return;
     }
-    stagger_start(3);
     if (ch.groups == 1) fc2_body<1>(a, ch, ob, lane);
     else if (ch.groups == 2) fc2_body<2>(a, ch, ob, lane);
     else if (ch.groups <= 4) fc2_tile_body<4>(a, ch, c, ob, wv, lane, lds);
