@@ -23,6 +23,11 @@ sys.path.insert(0, os.path.join(ROOT, "oracle"))
 
 HBM_PEAK_GBS = 8000.0           # MI355X HBM3E, published
 MFMA_FP8_PEAK_TFLOPS = 5000.0   # dense FP8 (an FP8 x FP4 block-scaled MFMA issues at the FP8 rate)
+# HBM bytes per launch of the dominant kernels on these workloads, from two rocprofv3 --pmc runs of this
+# file (FETCH_SIZE, WRITE_SIZE), each scaled by what the same counter reads for --copy-probe's 1 GiB copy:
+# one FETCH_SIZE count = 2.0 KiB, one WRITE_SIZE count = 1.0 KiB.
+FC1_DECODE_TRAFFIC_BYTES = int((2.0 * 858260 + 1.0 * 2567) * 1024)
+FC1_PREFILL_TRAFFIC_BYTES = int((2.0 * 2754783 + 1.0 * 141470) * 1024)
 
 
 def log(*a):
@@ -134,6 +139,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-prefill", action="store_true", help="skip the 8192-token prefill measurement")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="profiling aid: also run a 1 GiB -> 1 GiB elementwise copy (torch add), the kernel of known "
+                         "size that scales the FETCH_SIZE / WRITE_SIZE counters")
     ap.add_argument("--only-prefill", action="store_true",
                     help="profiling aid: run only the prefill measurement and print its object")
     args = ap.parse_args()
@@ -148,6 +156,14 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
 
+    if args.copy_probe:
+        src = torch.zeros(1 << 28, dtype=torch.int32, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            torch.add(src, 1, out=dst)
+        torch.cuda.synchronize()
+        del src, dst
+        torch.cuda.empty_cache()
     if args.only_prefill:
         pre = run_config(3, args.steps, args.warmup, torch, dev, b1, synth, O, parity_tokens=2, cpu_tokens=0)
         print(json.dumps(dict(ms_per_step=pre["ms_per_step"], phases=pre["phases"], parity=pre["parity"])), flush=True)
@@ -174,7 +190,7 @@ def main():
                    "activations": "bf16 N(0,1) -> wire quantizer FP8 e4m3 + ue8m0/32"},
         "roofline": {"bound": "hbm", "kernel": "fc1_kernel<2> (gate/up GEMM + SwiGLU + requant)",
                      "achieved": fc1_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": fc1_gbs / HBM_PEAK_GBS,
-                     "traffic": None, "algorithmic_bytes": fc1_bytes, "kernel_ms": dec["phases"]["fc1_ms"],
+                     "traffic": FC1_DECODE_TRAFFIC_BYTES, "algorithmic_bytes": fc1_bytes, "kernel_ms": dec["phases"]["fc1_ms"],
                      "path": {"algorithmic_bytes": path_bytes, "achieved": path_gbs, "frac": path_gbs / HBM_PEAK_GBS,
                               "plan_ms": dec["phases"]["plan_ms"], "fc2_ms": dec["phases"]["fc2_ms"],
                               "reduce_ms": dec["phases"]["reduce_ms"], "event_ms_per_step": dec["event_ms_per_step"]}},
@@ -194,7 +210,7 @@ def main():
             "value": pw.rows / (pre["ms_per_step"] * 1e-3), "unit": "routed tok/s per MoE layer",
             "ms_per_step": pre["ms_per_step"], "steps": max(3, args.steps // 5),
             "roofline": {"bound": "mfma", "kernel": "fc1_tile_kernel (gate/up GEMM + SwiGLU + requant)", "achieved": fc1_tf, "peak": MFMA_FP8_PEAK_TFLOPS,
-                         "unit": "TFLOP/s", "frac": fc1_tf / MFMA_FP8_PEAK_TFLOPS, "traffic": None,
+                         "unit": "TFLOP/s", "frac": fc1_tf / MFMA_FP8_PEAK_TFLOPS, "traffic": FC1_PREFILL_TRAFFIC_BYTES,
                          "algorithmic_flops": fc1_flops, "kernel_ms": pre["phases"]["fc1_ms"],
                          "path": {"algorithmic_flops": flops, "achieved": tf, "frac": tf / MFMA_FP8_PEAK_TFLOPS,
                                   "plan_ms": pre["phases"]["plan_ms"], "fc2_ms": pre["phases"]["fc2_ms"],
