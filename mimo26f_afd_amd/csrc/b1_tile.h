@@ -271,6 +271,15 @@ __device__ __forceinline__ void gemm_chunk_lds(v4f (&acc)[4][TT], const uint8_t*
 #undef M26G_QUAD
 #undef M26G_KSTEP
     wait_loads_but<0>();  // the re-staged tail loads must land before the LDS is reused or the wave ends
+    wait_lds_but<0>();
+    // The last fetches of scales, fragment and weights feed no MFMA. To the compiler such a register is
+    // free the moment the load has issued, and whatever it puts there next is overwritten when the
+    // data lands. Naming them here keeps them reserved until the waits above have passed.
+#pragma unroll
+    for (int t = 0; t < 4; ++t) asm volatile("" ::"v"(sw0[t]), "v"(sw1[t]), "v"(af[0][t]), "v"(af[1][t]));
+#pragma unroll
+    for (int tt = 0; tt < TT; ++tt) asm volatile("" ::"v"(sa0[tt]), "v"(sa1[tt]));
+    asm volatile("" ::"v"(flo), "v"(fhi));
     // The MFMAs above are opaque to the compiler's hazard tracking: let the last ones retire before
     // the epilogue reads the accumulators (8 passes of 4 cycles, plus margin).
     asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15" ::: "memory");

@@ -144,6 +144,26 @@ def test_rank_share_configs(scratch, cfg):
     assert np.array_equal(out2, bf)
 
 
+def test_tile_schedule_at_rank_share_stage_by_stage(scratch):
+    """More than 512 rows at one rank's share (I = 512): the prefill schedule with chunks of every class
+    (1, 2, 3-4 and 5-8 groups under Zipf routing) and an FC2 of a single quad of k-steps, checked stage
+    by stage like the decode configurations: plan, gate/up/h taps, codec bytes, per-route rows, outputs."""
+    rows, seed = 1200, synth.BASE_SEED + 7
+    ids, w, x = synth.routes_zipf(seed, rows), synth._softmax_weights(seed, rows), synth._activations(seed, rows)
+    payload, scales = synth.q0_quantize(x)
+    wl = synth.Workload("tile schedule, rank share", 1, seed, 1, rows, ids, w, x, payload, scales)
+    groups_of = (np.bincount(ids.reshape(-1), minlength=256) + 15) // 16
+    assert (groups_of == 1).any() and (groups_of == 2).any() and ((groups_of % 8 == 3) | (groups_of % 8 == 4)).any() \
+        and (groups_of >= 5).any()
+    pools = wl.pools(wl.touched())
+    layer = DeviceLayer(pools).layer
+    stats, bf, pf = run_ffn_dev(layer, scratch, wl)
+    rc, ref_partial, ref_bf16, _ = O.layer_ffn(pools, wl.payload, wl.scales, wl.ids, wl.weights)
+    assert rc == 0
+    check_outputs(pf, bf, ref_partial, ref_bf16)
+    check_stages(scratch, layer, wl, pools, stats, experts=12)
+
+
 @pytest.fixture(scope="module")
 def full_layer():
     wl = synth.make(2)
