@@ -1,0 +1,94 @@
+// C ABI of the coordinator-side kernels (include/m26c_glue.h): argument checks and launches.
+#include "../../include/m26c_glue.h"
+#include "glue_kernels.h"
+
+namespace {
+
+using namespace m26g;
+
+constexpr int kThreads = 256;
+
+int grid_for(long n) {
+    long g = (n + kThreads - 1) / kThreads;
+    if (g > 65535L * 8) g = 65535L * 8;
+    return int(g < 1 ? 1 : g);
+}
+
+int launched() { return int(hipGetLastError()); }
+
+}  // namespace
+
+extern "C" {
+
+int m26c_router_topk(const float* logits, const float* bias, int rows, int n_experts, int top_k, int* idx_out,
+                     float* w_out, void* stream) {
+    if (rows <= 0) return 0;
+    if (n_experts <= 0 || n_experts > 64 * kRouterPerLane || n_experts % 32 || top_k <= 0 || top_k > n_experts ||
+        top_k > 64 || !logits || !bias || !idx_out || !w_out)
+        return 1;
+    router_topk_kernel<<<(rows + 3) / 4, kThreads, 0, hipStream_t(stream)>>>(logits, bias, rows, n_experts, top_k, idx_out,
+                                                                            w_out);
+    return launched();
+}
+
+int m26c_quant_scales(const float* x, long n_blocks, unsigned char* scales, float* scale_inv, void* stream) {
+    if (n_blocks <= 0) return 0;
+    if (!x || !scales || !scale_inv) return 1;
+    quantize_hidden_kernel<<<grid_for(n_blocks * 8), kThreads, 0, hipStream_t(stream)>>>(x, n_blocks, 32, nullptr, 0, scales, 1,
+                                                                                        scale_inv);
+    return launched();
+}
+
+int m26_quantize_hidden_fp8(const float* x, const float* scale_inv, uint8_t* payload, int64_t n_elem, void* stream) {
+    if (n_elem <= 0) return 0;
+    if (!x || !scale_inv || !payload) return 1;
+    encode_hidden_kernel<<<grid_for(long((n_elem + 3) / 4)), kThreads, 0, hipStream_t(stream)>>>(x, scale_inv, payload, n_elem);
+    return launched();
+}
+
+int m26c_quantize_hidden(const float* x, long rows, int cols, uint8_t* payload, size_t payload_pitch, uint8_t* scales,
+                         size_t scales_pitch, void* stream) {
+    if (rows <= 0) return 0;
+    if (!x || !payload || !scales || cols <= 0 || cols % 32 || payload_pitch < size_t(cols) || scales_pitch < size_t(cols / 32) ||
+        payload_pitch % 4)
+        return 1;
+    quantize_hidden_kernel<<<grid_for(rows * (cols / 32) * 8), kThreads, 0, hipStream_t(stream)>>>(
+        x, rows, cols, payload, payload_pitch, scales, scales_pitch, nullptr);
+    return launched();
+}
+
+int m26c_frame_fill(const int* idx, const float* wts, const uint8_t* payload, const uint8_t* scales, int t, int topk,
+                    int hid, uint8_t* routes, uint8_t* hidden, int pitch, void* stream) {
+    if (t <= 0) return 0;
+    if (!idx || !wts || !payload || !scales || !routes || !hidden || topk <= 0 || hid <= 0 || hid % 256 ||
+        pitch < hid + hid / 32 || pitch % 8)
+        return 1;
+    const long n = long(t) * topk + long(t) * (hid / 8 + hid / 32 / 8);
+    frame_fill_kernel<<<grid_for(n), kThreads, 0, hipStream_t(stream)>>>(idx, wts, payload, scales, t, topk, hid, routes, hidden,
+                                                                        pitch);
+    return launched();
+}
+
+int m26c_rank_sum_bf16(const uint16_t* p0, const uint16_t* p1, const uint16_t* p2, const uint16_t* p3, float* out,
+                       long n, void* stream) {
+    if (n <= 0) return 0;
+    if (!p0 || !p1 || !p2 || !p3 || !out) return 1;
+    rank_sum_bf16_kernel<<<grid_for(n), kThreads, 0, hipStream_t(stream)>>>(p0, p1, p2, p3, out, n);
+    return launched();
+}
+
+int m26c_add_inplace(float* h, const float* a, long n, void* stream) {
+    if (n <= 0) return 0;
+    if (!h || !a) return 1;
+    add_inplace_kernel<<<grid_for(n), kThreads, 0, hipStream_t(stream)>>>(h, a, n);
+    return launched();
+}
+
+int m26c_f32_to_bf16(const float* x, uint16_t* y, long n, void* stream) {
+    if (n <= 0) return 0;
+    if (!x || !y) return 1;
+    f32_to_bf16_kernel<<<grid_for(n), kThreads, 0, hipStream_t(stream)>>>(x, y, n);
+    return launched();
+}
+
+}  // extern "C"

@@ -27,6 +27,14 @@
  *                         identity, M-prefix identity and mutation detectors.
  *   orc_layer_ffn_efp32 - structure check only against the W4A8 path (same routing, looser
  *                         numerics); it is a reported baseline, not a parity oracle.
+ *   orc_router_topk     - the reference holds no vectors for it: a stable argsort of library
+ *                         sigmoids (scipy expit), the tie rule on equal logits, bias selecting but
+ *                         not weighting, a closed-form two-expert weight.
+ *   orc_q0_scales       - closed form on amax = 448 * 2^e and its neighbours over the whole
+ *                         exponent range, identity with orc_q0_quantize's scale bytes.
+ *   orc_rank_sum_bf16   - sequential binary32 additions in numpy, data where another order
+ *                         differs, and the 1 + 2^-24 + 2^-24 - 1 case a fused sum gets wrong.
+ *   orc_bf16_rne_nan    - midpoint, signed-zero, infinity, NaN and subnormal vectors.
  */
 #include "b1_oracle.h"
 #include <float.h>
@@ -578,3 +586,59 @@ uint32_t orc_layer_ffn_efp32(const orc_layer* layer, const uint8_t* x_payload, s
     (void)threads;
     return 0;
 }
+
+/* ------------------------------------------------------------------------------------------
+ * Coordinator-side steps around the path
+ * ---------------------------------------------------------------------------------------- */
+
+/* crates/mimo26-coordinator/src/router.rs:41-80: scores = 1 / (1 + exp(-logit)) in FP64; order by
+ * score + bias descending, stable over ascending ids; weights from the unbiased scores. */
+void orc_router_topk(const float* logits, const float* bias, size_t rows, size_t n_experts, size_t top_k,
+                     int32_t* idx, float* weights) {
+    double* score = (double*)malloc(n_experts * sizeof(double));
+    double* sel = (double*)malloc(n_experts * sizeof(double));
+    for (size_t r = 0; r < rows; ++r) {
+        for (size_t e = 0; e < n_experts; ++e) {
+            score[e] = 1.0 / (1.0 + exp(-(double)logits[r * n_experts + e]));
+            sel[e] = score[e] + (double)bias[e];
+        }
+        double wsum = 0.0;
+        for (size_t k = 0; k < top_k; ++k) { /* k passes of "largest remaining, lowest id first" = stable sort prefix */
+            size_t best = n_experts;
+            for (size_t e = 0; e < n_experts; ++e)
+                if (!isnan(sel[e]) && (best == n_experts || sel[e] > sel[best])) best = e;
+            idx[r * top_k + k] = (int32_t)best;
+            wsum += score[best];
+            sel[best] = NAN; /* taken */
+        }
+        for (size_t k = 0; k < top_k; ++k) weights[r * top_k + k] = (float)(score[idx[r * top_k + k]] / wsum);
+    }
+    free(score);
+    free(sel);
+}
+
+/* crates/mimo26-coordinator/src/wire.rs:83-108: the scale half of orc_q0_quantize and the power of
+ * two the payload half multiplies by. */
+void orc_q0_scales(const float* x, size_t n_blocks, uint8_t* scales, float* scale_inv) {
+    for (size_t b = 0; b < n_blocks; ++b) {
+        uint8_t s;
+        uint8_t scratch[32];
+        orc_q0_quantize(x + b * 32, 1, 32, scratch, &s);
+        scales[b] = s;
+        scale_inv[b] = ldexpf(1.0f, 127 - (int)s);
+    }
+}
+
+/* crates/mimo26-wire/src/l4.rs (CoordinatorSum), crates/mimo26-coordinator/kernels/glue.cu:198-213. */
+void orc_rank_sum_bf16(const uint16_t* p0, const uint16_t* p1, const uint16_t* p2, const uint16_t* p3,
+                       float* out, size_t n) {
+    const uint16_t* p[4] = {p0, p1, p2, p3};
+    for (size_t i = 0; i < n; ++i) {
+        volatile float s = 0.0f; /* one rounding per addition, no contraction */
+        for (int r = 0; r < 4; ++r) s = s + bits_f32((uint32_t)p[r][i] << 16);
+        out[i] = s;
+    }
+}
+
+uint16_t orc_bf16_rne_nan(float v) { return isnan(v) ? (uint16_t)0x7fff : orc_bf16_rne(v); }
+

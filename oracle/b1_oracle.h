@@ -117,6 +117,21 @@ uint32_t orc_layer_ffn_efp32(const orc_layer* layer, const uint8_t* x_payload, s
 
 int orc_hardware_threads(void);
 
+/* ---- coordinator-side steps around the path ------------------------------------------------- */
+
+/* Router selection over FP32 logits [rows][n_experts]: FP64 sigmoid, top_k by (score + bias)
+ * descending with ties to the lower expert id, weights = unbiased scores over their sum taken in
+ * selection order (FP64), rounded to FP32. */
+void orc_router_topk(const float* logits, const float* bias, size_t rows, size_t n_experts, size_t top_k,
+                     int32_t* idx, float* weights);
+/* Q0's scale half: scale byte and 2^(127 - s) per K32 block. */
+void orc_q0_scales(const float* x, size_t n_blocks, uint8_t* scales, float* scale_inv);
+/* out = ((((0 + p0) + p1) + p2) + p3) over BF16 values, FP32 additions in that order. */
+void orc_rank_sum_bf16(const uint16_t* p0, const uint16_t* p1, const uint16_t* p2, const uint16_t* p3,
+                       float* out, size_t n);
+/* FP32 -> BF16 round to nearest even, NaN -> 0x7fff (the conversion the reference's GEMM input cast uses). */
+uint16_t orc_bf16_rne_nan(float v);
+
 #ifdef __cplusplus
 }
 #endif

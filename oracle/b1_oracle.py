@@ -55,6 +55,8 @@ def _load():
     lib.orc_layer_ffn.restype = C.c_uint32
     lib.orc_layer_ffn_efp32.restype = C.c_uint32
     lib.orc_hardware_threads.restype = C.c_int
+    lib.orc_bf16_rne_nan.restype = C.c_uint16
+    lib.orc_bf16_rne_nan.argtypes = [C.c_float]
     return lib
 
 
@@ -101,6 +103,38 @@ def q0_quantize(x: np.ndarray):
     scales = np.empty((rows, cols // 32), np.uint8)
     LIB.orc_q0_quantize(_p(x, _f32p), C.c_size_t(rows), C.c_size_t(cols), _p(payload, _u8p), _p(scales, _u8p))
     return payload, scales
+
+
+def q0_scales(x: np.ndarray):
+    """Scale bytes and 2^(127 - s) per K32 block of a flat f32 array."""
+    x = np.ascontiguousarray(x, np.float32).reshape(-1)
+    n = x.size // 32
+    scales, inv = np.empty(n, np.uint8), np.empty(n, np.float32)
+    LIB.orc_q0_scales(_p(x, _f32p), C.c_size_t(n), _p(scales, _u8p), _p(inv, _f32p))
+    return scales, inv
+
+
+def router_topk(logits: np.ndarray, bias: np.ndarray, top_k: int):
+    logits = np.ascontiguousarray(logits, np.float32)
+    bias = np.ascontiguousarray(bias, np.float32)
+    rows, n = logits.shape
+    idx, w = np.empty((rows, top_k), np.int32), np.empty((rows, top_k), np.float32)
+    LIB.orc_router_topk(_p(logits, _f32p), _p(bias, _f32p), C.c_size_t(rows), C.c_size_t(n), C.c_size_t(top_k),
+                        _p(idx, C.POINTER(C.c_int32)), _p(w, _f32p))
+    return idx, w
+
+
+def rank_sum_bf16(p0, p1, p2, p3) -> np.ndarray:
+    ps = [np.ascontiguousarray(p, np.uint16).reshape(-1) for p in (p0, p1, p2, p3)]
+    out = np.empty(ps[0].size, np.float32)
+    u16p = C.POINTER(C.c_uint16)
+    LIB.orc_rank_sum_bf16(*[_p(p, u16p) for p in ps], _p(out, _f32p), C.c_size_t(out.size))
+    return out
+
+
+def bf16_rne_nan(x: np.ndarray) -> np.ndarray:
+    x = np.ascontiguousarray(x, np.float32).reshape(-1)
+    return np.array([LIB.orc_bf16_rne_nan(C.c_float(float(v))) for v in x], np.uint16)
 
 
 def quant_v1(h: np.ndarray, fill: int = 0xA5):

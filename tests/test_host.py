@@ -15,9 +15,12 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
 def declared_symbols():
-    text = open(os.path.join(ROOT, "include", "m26s_b1.h")).read()
-    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    return sorted(set(re.findall(r"\b(m26s_b1_\w+)\s*\(", text)))
+    names = set()
+    for header in ("m26s_b1.h", "m26c_glue.h"):
+        text = open(os.path.join(ROOT, "include", header)).read()
+        text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+        names |= set(re.findall(r"\b(m26s_b1_\w+|m26c?_\w+)\s*\(", text))
+    return sorted(names)
 
 
 def test_library_exports_every_declared_symbol():
@@ -25,9 +28,9 @@ def test_library_exports_every_declared_symbol():
         build.build_library()
     lib = ctypes.CDLL(build.LIB)
     names = declared_symbols()
-    assert len(names) >= 20
+    assert len(names) >= 29
     for name in names:
-        assert hasattr(lib, name), f"{name} declared in include/m26s_b1.h but not exported"
+        assert hasattr(lib, name), f"{name} declared in include/*.h but not exported"
     assert sorted(_lib.SIGNATURES) == names  # the Python binding covers the same set
 
 
