@@ -374,18 +374,21 @@ __global__ void __launch_bounds__(256) quantize_kernel(const float* __restrict__
 // The walk over K starts at quad `first` and wraps, so waves that stream neighbouring weight
 // blocks do not sit on the same addresses modulo the block size at the same time.
 // ---------------------------------------------------------------------------------------------
+// Weight fragments of one k-step (four tiles) and the activation fragments of one k-step.
+struct WeightStep { v4i a[4]; };
 template <int TT>
-struct Operands {
-    v4i a[4];
+struct ActStep {
     v4i lo[TT], hi[TT];
     uint32_t sb[TT];
 };
 
-template <int TT>
-__device__ __forceinline__ void load_step(Operands<TT>& o, const uint8_t* __restrict__ wp, int ks,
-                                          const uint8_t* const (&xrow)[TT], const uint8_t* const (&xsrow)[TT]) {
+__device__ __forceinline__ void load_weights(WeightStep& o, const uint8_t* __restrict__ wp, int ks) {
 #pragma unroll
     for (int t = 0; t < 4; ++t) o.a[t] = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(wp + size_t(ks) * 4096 + t * 1024));
+}
+template <int TT>
+__device__ __forceinline__ void load_acts(ActStep<TT>& o, int ks, const uint8_t* const (&xrow)[TT],
+                                          const uint8_t* const (&xsrow)[TT]) {
 #pragma unroll
     for (int tt = 0; tt < TT; ++tt) {
         o.lo[tt] = *reinterpret_cast<const v4i*>(xrow[tt] + ks * 128);
@@ -395,16 +398,16 @@ __device__ __forceinline__ void load_step(Operands<TT>& o, const uint8_t* __rest
 }
 
 template <int TT, int SEL>
-__device__ __forceinline__ void mfma_step(v4f (&acc)[4][TT], const Operands<TT>& o, const uint32_t (&sw)[4],
-                                          uint32_t shift, uint32_t& bad) {
+__device__ __forceinline__ void mfma_step(v4f (&acc)[4][TT], const WeightStep& w, const ActStep<TT>& x,
+                                          const uint32_t (&sw)[4], uint32_t shift, uint32_t& bad) {
 #pragma unroll
     for (int tt = 0; tt < TT; ++tt) {
-        const uint32_t s = (o.sb[tt] >> shift) & 0xffu;
+        const uint32_t s = (x.sb[tt] >> shift) & 0xffu;
         bad |= (s - 105u) > 142u ? 1u : 0u;  // activation scales are legal only in [105, 247]
-        const v8i b = {o.lo[tt].x, o.lo[tt].y, o.lo[tt].z, o.lo[tt].w, o.hi[tt].x, o.hi[tt].y, o.hi[tt].z, o.hi[tt].w};
+        const v8i b = {x.lo[tt].x, x.lo[tt].y, x.lo[tt].z, x.lo[tt].w, x.hi[tt].x, x.hi[tt].y, x.hi[tt].z, x.hi[tt].w};
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
-            const v8i a = {o.a[t].x, o.a[t].y, o.a[t].z, o.a[t].w, 0, 0, 0, 0};
+            const v8i a = {w.a[t].x, w.a[t].y, w.a[t].z, w.a[t].w, 0, 0, 0, 0};
             acc[t][tt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, acc[t][tt], 4 /*A: E2M1*/,
                                                                           0 /*B: E4M3*/, SEL, int(sw[t]), 0, int(s));
         }
@@ -412,31 +415,47 @@ __device__ __forceinline__ void mfma_step(v4f (&acc)[4][TT], const Operands<TT>&
 }
 
 // wp / sp already include the lane offset (lane*16, lane*4). ksteps is a multiple of 4.
+//
+// This is the schedule of the HBM-bound sizes, so what counts is bytes in flight: the weight stream
+// (4 KB per wave and k-step, each byte used once) runs three k-steps ahead of the MFMAs in a ring of
+// four register sets, about 12 KB per wave and 36 KB per SIMD at three waves, which is what 7 TB/s
+// times the memory latency asks for. Activation rows come from L2 and run one k-step ahead; the
+// weight scale dwords of the next quad of k-steps are fetched a quad ahead. Past the end the last
+// k-step is fetched again rather than branching.
 template <int TT>
 __device__ __forceinline__ void gemm_chunk(v4f (&acc)[4][TT], const uint8_t* __restrict__ wp,
-                                           const uint8_t* __restrict__ sp, int ksteps, int first,
+                                           const uint8_t* __restrict__ sp, int ksteps,
                                            const uint8_t* const (&xrow)[TT], const uint8_t* const (&xsrow)[TT],
                                            uint32_t lane, uint32_t& bad) {
     const uint32_t shift = 8 * (lane >> 4);
-    const int quads = ksteps / 4;
-    Operands<TT> cur, nxt;
-    int q = first;
-    load_step<TT>(cur, wp, 4 * q, xrow, xsrow);
-    for (int i = 0; i < quads; ++i) {
-        uint32_t sw[4];
+    const int quads = ksteps / 4, last = ksteps - 1;
+    WeightStep w[4];
+    ActStep<TT> x[2];
+    uint32_t sw[4], swn[4];
+    load_weights(w[0], wp, 0);
+    load_weights(w[1], wp, 1);
+    load_weights(w[2], wp, 2);
+    load_acts<TT>(x[0], 0, xrow, xsrow);
 #pragma unroll
-        for (int t = 0; t < 4; ++t) sw[t] = *reinterpret_cast<const uint32_t*>(sp + size_t(q) * 1024 + t * 256);
-        const int ks = 4 * q;
-        const int qn = q + 1 == quads ? 0 : q + 1;
-        load_step<TT>(nxt, wp, ks + 1, xrow, xsrow);
-        mfma_step<TT, 0>(acc, cur, sw, shift, bad);
-        load_step<TT>(cur, wp, ks + 2, xrow, xsrow);
-        mfma_step<TT, 1>(acc, nxt, sw, shift, bad);
-        load_step<TT>(nxt, wp, ks + 3, xrow, xsrow);
-        mfma_step<TT, 2>(acc, cur, sw, shift, bad);
-        if (i + 1 < quads) load_step<TT>(cur, wp, 4 * qn, xrow, xsrow);
-        mfma_step<TT, 3>(acc, nxt, sw, shift, bad);
-        q = qn;
+    for (int t = 0; t < 4; ++t) sw[t] = *reinterpret_cast<const uint32_t*>(sp + t * 256);
+    for (int q = 0; q < quads; ++q) {
+        const int ks = 4 * q, qn = q + 1 < quads ? q + 1 : q;
+#pragma unroll
+        for (int t = 0; t < 4; ++t) swn[t] = *reinterpret_cast<const uint32_t*>(sp + size_t(qn) * 1024 + t * 256);
+        load_weights(w[3], wp, ks + 3);
+        load_acts<TT>(x[1], ks + 1, xrow, xsrow);
+        mfma_step<TT, 0>(acc, w[0], x[0], sw, shift, bad);
+        load_weights(w[0], wp, ks + 4 < last ? ks + 4 : last);
+        load_acts<TT>(x[0], ks + 2, xrow, xsrow);
+        mfma_step<TT, 1>(acc, w[1], x[1], sw, shift, bad);
+        load_weights(w[1], wp, ks + 5 < last ? ks + 5 : last);
+        load_acts<TT>(x[1], ks + 3, xrow, xsrow);
+        mfma_step<TT, 2>(acc, w[2], x[0], sw, shift, bad);
+        load_weights(w[2], wp, ks + 6 < last ? ks + 6 : last);
+        load_acts<TT>(x[0], ks + 4 < last ? ks + 4 : last, xrow, xsrow);
+        mfma_step<TT, 3>(acc, w[3], x[1], sw, shift, bad);
+#pragma unroll
+        for (int t = 0; t < 4; ++t) sw[t] = swn[t];
     }
 }
 
@@ -596,7 +615,7 @@ __device__ __forceinline__ void fc1_body(const Fc1Args& a, const Chunk ch, uint3
 #pragma unroll
         for (int tt = 0; tt < TT; ++tt) acc[t][tt] = v4f{0.f, 0.f, 0.f, 0.f};
     uint32_t bad = 0;
-    gemm_chunk<TT>(acc, wp, sp, 32, 0, xrow, xsrow, lane, bad);
+    gemm_chunk<TT>(acc, wp, sp, 32, xrow, xsrow, lane, bad);
     fc1_finish<TT>(a, ch, cb, lane, acc, bad, live);
 }
 
@@ -679,7 +698,7 @@ __device__ __forceinline__ void fc2_body(const Fc2Args& a, const Chunk ch, uint3
 #pragma unroll
         for (int tt = 0; tt < TT; ++tt) acc[t][tt] = v4f{0.f, 0.f, 0.f, 0.f};
     uint32_t bad = 0;
-    gemm_chunk<TT>(acc, wp, sp, int(ksteps), 0, xrow, xsrow, lane, bad);
+    gemm_chunk<TT>(acc, wp, sp, int(ksteps), xrow, xsrow, lane, bad);
     fc2_finish<TT>(a, ob, lane, acc, route);
 }
 
