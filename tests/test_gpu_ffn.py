@@ -145,7 +145,7 @@ def test_rank_share_configs(scratch, cfg):
 
 
 def test_tile_schedule_at_rank_share_stage_by_stage(scratch):
-    """More than 512 rows at one rank's share (I = 512): the prefill schedule with chunks of every class
+    """More than 128 rows at one rank's share (I = 512): the prefill schedule with chunks of every class
     (1, 2, 3-4 and 5-8 groups under Zipf routing) and an FC2 of a single quad of k-steps, checked stage
     by stage like the decode configurations: plan, gate/up/h taps, codec bytes, per-route rows, outputs."""
     rows, seed = 1200, synth.BASE_SEED + 7
