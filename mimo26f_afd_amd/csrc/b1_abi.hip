@@ -222,7 +222,7 @@ int enqueue(const m26s_b1_layer* L, m26s_b1_scratch* S, const uint8_t* x, size_t
     else launch_tiles(L, S, pv, x, xp, xs, xsp, uint32_t(ccap), routes);
     M26S_CK(hipGetLastError(), "b1 fc launch");
     const uint64_t n4 = uint64_t(rows) * (kHidden / 4);
-    const uint32_t blocks = uint32_t(n4 / 256 < 8192 ? (n4 + 255) / 256 : 8192);
+    const uint32_t blocks = uint32_t(n4 / 256 < 65536 ? (n4 + 255) / 256 : 65536);
     reduce_kernel<<<blocks, 256, 0, S->st>>>(S->y.as<float>(), w, rows, partial, bf16_out,
                                              S->meta.as<uint32_t>() + kReduceFault, S->meta.as<uint32_t>());
     M26S_CK(hipGetLastError(), "b1 reduce launch");
@@ -452,7 +452,7 @@ int m26s_b1_reduce_dev(const float* y_dev, const float* weights_dev, uint32_t ro
     M26S_CK(hipMemset(fault_dev, 0, 4), "b1 reduce fault clear");
     if (!rows) return 0;
     const uint64_t n4 = uint64_t(rows) * (kHidden / 4);
-    reduce_kernel<<<uint32_t(n4 / 256 < 8192 ? (n4 + 255) / 256 : 8192), 256>>>(y_dev, weights_dev, rows, partial_dev,
+    reduce_kernel<<<uint32_t(n4 / 256 < 65536 ? (n4 + 255) / 256 : 65536), 256>>>(y_dev, weights_dev, rows, partial_dev,
                                                                                 bf16_dev, fault_dev, nullptr);
     M26S_CK(hipGetLastError(), "b1 reduce launch");
     M26S_CK(hipDeviceSynchronize(), "b1 reduce sync");
