@@ -52,6 +52,7 @@ uint64_t chunk_bound(uint64_t routes, uint32_t gpc) {
 // weights for up to 32 rows; larger calls reuse each weight fragment over 128 rows. The tile schedule
 // runs small chunks through the same register-only bodies, and measured from 192 rows up it is never
 // slower than the direct one (Zipf routing: 0.51 against 0.53 ms at 192 rows, 0.62 against 0.67 at 384).
+constexpr uint32_t kWidePlanFrom = 512;  // rows above which the planner runs on several compute units
 uint32_t tiles_for(uint32_t rows) { return rows <= 32 ? 1u : rows <= 128 ? 2u : 8u; }
 
 // Kernels whose dynamic LDS passes 64 KB need the limit raised once per process.
@@ -83,7 +84,7 @@ struct m26s_b1_scratch {
     hipStream_t st = nullptr;
     bool own_stream = false;
     hipEvent_t e0 = nullptr, ep = nullptr, ea = nullptr, ec = nullptr, e1 = nullptr;
-    Dev x, xs, iw, inv, orig, gw, groups, chunks, meta, dq, dqs, y, bf16, pad, tap_gate, tap_up, tap_h, xg, rowbad, dg;
+    Dev x, xs, iw, inv, orig, gw, groups, chunks, meta, dq, dqs, y, bf16, pad, tap_gate, tap_up, tap_h, xg, rowbad, dg, planw;
     std::vector<uint8_t> hiw;
     bool taps = false;
     uint32_t last_rows = 0, last_inter = 0;
@@ -214,7 +215,17 @@ int enqueue(const m26s_b1_layer* L, m26s_b1_scratch* S, const uint8_t* x, size_t
                       S->chunks.as<Chunk>(), S->meta.as<uint32_t>()};
     M26S_CK(hipEventRecord(S->e0, S->st), "b1 event 0");
     // Stage faults accumulate across enqueued calls until the next sync; only the plan words reset.
-    plan_kernel<<<1, kPlanThreads, routes, S->st>>>(ids, w, rows, L->resident, pv, nt, 0, S->taps);
+    if (rows > kWidePlanFrom) {  // several compute units share the scatter (b1_kernels.h, "Stage 1 for large calls")
+        const void* before = S->planw.p;
+        M26S_CK(S->planw.ensure(wide_plan_words(uint32_t(route_cap)) * 4), "b1 plan work alloc");
+        if (S->planw.p != before) M26S_CK(hipMemsetAsync(S->planw.p, 0xff, 16, S->st), "b1 plan work arm");  // a new buffer: no fault yet
+        const uint32_t wide = wide_plan_groups(uint32_t(routes));
+        plan_count_kernel<<<wide, kPlanThreads, 0, S->st>>>(ids, w, rows, L->resident, S->planw.as<uint32_t>());
+        plan_scan_kernel<<<1, kPlanThreads, 0, S->st>>>(uint32_t(routes), S->planw.as<uint32_t>(), pv, nt);
+        plan_place_kernel<<<wide, kPlanThreads, 0, S->st>>>(ids, w, rows, S->planw.as<uint32_t>(), pv, S->taps);
+    } else {
+        plan_kernel<<<1, kPlanThreads, routes, S->st>>>(ids, w, rows, L->resident, pv, nt, 0, S->taps);
+    }
     M26S_CK(hipGetLastError(), "b1 plan launch");
     M26S_CK(hipEventRecord(S->ep, S->st), "b1 event p");
     if (nt == 1) launch_ffn<1>(L, S, pv, x, xp, xs, xsp, uint32_t(ccap), routes);

@@ -300,6 +300,199 @@ plan_kernel(const int32_t* __restrict__ ids, const float* __restrict__ w, uint32
     }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Stage 1 for large calls: the same stable counting sort spread over several compute units.
+//
+// One workgroup scatters its results through one memory pipeline; at 65536 routes the placement's
+// three uncoalesced stores per route kept that pipeline busy for 0.1 ms. Here a wave still owns one
+// contiguous run of routes (256 of them: wave w of all workgroups taken together owns routes
+// [256 w, 256 w + 256)), so the order inside an expert is the serial planner's, and the work is cut
+// into three launches on the stream:
+//   plan_count_kernel  validates, and leaves every wave's per-expert counts in `work`;
+//   plan_scan_kernel   (one workgroup) turns them into every wave's first position inside each
+//                      expert, scans experts into route / group / chunk bases, fills group headers
+//                      and chunks, publishes the counts or the fault;
+//   plan_place_kernel  walks the routes again and places them.
+// work: [0] first fault key (0xffffffff = none; the scan re-arms it), [1..3] unused,
+//       [4 ..) counts[wave][256], then route and group bases [2][257].
+// ---------------------------------------------------------------------------------------------
+constexpr uint32_t kWideRoutesPerWave = 256, kWideRoutesPerGroup = kPlanWaves * kWideRoutesPerWave;
+__host__ __device__ constexpr uint32_t wide_plan_groups(uint32_t routes) { return (routes + kWideRoutesPerGroup - 1) / kWideRoutesPerGroup; }
+__host__ __device__ constexpr uint64_t wide_plan_words(uint32_t routes) {
+    return 4 + uint64_t(wide_plan_groups(routes)) * kPlanWaves * 256 + 2 * 257;
+}
+
+__global__ void __launch_bounds__(kPlanThreads)
+plan_count_kernel(const int32_t* __restrict__ ids, const float* __restrict__ w, uint32_t rows,
+                  const uint8_t* __restrict__ resident, uint32_t* __restrict__ work) {
+    __shared__ __align__(16) uint8_t id_byte[kWideRoutesPerGroup];
+    __shared__ uint32_t hist[kPlanWaves][256];
+    __shared__ uint8_t present[256];
+    const uint32_t tid = threadIdx.x, lane = tid & 63, wv = tid >> 6, routes = rows * kTopk;
+    const uint32_t first_route = blockIdx.x * kWideRoutesPerGroup;
+    for (uint32_t i = tid; i < kPlanWaves * 256; i += kPlanThreads) (&hist[0][0])[i] = 0;
+    if (tid < 256) {
+        const uint8_t here = resident[tid];
+        if (here > 1 && blockIdx.x == 0) atomicMin(&work[0], 1u);
+        present[tid] = here;
+    }
+    __syncthreads();
+    const uint32_t t = first_route / kTopk + tid;  // one token per thread, the first half of the workgroup
+    if (tid < kWideRoutesPerGroup / kTopk && t < rows) {
+        typedef v4i __attribute__((aligned(4))) v4i_u;
+        typedef v4f __attribute__((aligned(4))) v4f_u;
+        const v4i ia = reinterpret_cast<const v4i_u*>(ids)[2 * t], ib = reinterpret_cast<const v4i_u*>(ids)[2 * t + 1];
+        const v4f wa = reinterpret_cast<const v4f_u*>(w)[2 * t], wb = reinterpret_cast<const v4f_u*>(w)[2 * t + 1];
+        const int32_t e8[8] = {ia.x, ia.y, ia.z, ia.w, ib.x, ib.y, ib.z, ib.w};
+        const float w8[8] = {wa.x, wa.y, wa.z, wa.w, wb.x, wb.y, wb.z, wb.w};
+        uint32_t packed[2] = {0, 0};
+#pragma unroll
+        for (uint32_t j = 0; j < 8; ++j) {
+            const int32_t e = e8[j];
+            uint32_t check = 0;
+            if (e < 0 || e >= int32_t(kExperts) || !present[e & 255]) check = 1;
+            else if (!(w8[j] >= 0.0f && w8[j] <= FLT_MAX)) check = 2;
+            if (check) atomicMin(&work[0], ((t * 8 + j + 1) << 4) | check);
+            packed[j >> 2] |= (uint32_t(e) & 0xffu) << (8 * (j & 3));
+        }
+        *reinterpret_cast<uint2*>(id_byte + tid * 8) = uint2{packed[0], packed[1]};
+    }
+    __syncthreads();
+#pragma unroll
+    for (uint32_t step = 0; step < kWideRoutesPerWave / 64; ++step) {
+        const uint32_t local = wv * kWideRoutesPerWave + step * 64 + lane, i = first_route + local;
+        const bool valid = i < routes;
+        const uint32_t e = valid ? id_byte[local] : 0;
+        const uint64_t m = same_expert_lanes(e, valid);
+        const uint64_t below = m & ((1ull << lane) - 1);
+        if (valid) {
+            if (below & (0xffull << (lane & ~7u))) atomicMin(&work[0], ((i + 1) << 4) | 3u);
+            if (!below) hist[wv][e] += __popcll(m);
+        }
+    }
+    uint32_t* mine = work + 4 + (uint64_t(blockIdx.x) * kPlanWaves + wv) * 256;
+#pragma unroll
+    for (uint32_t j = 0; j < 4; ++j) mine[lane + 64 * j] = hist[wv][lane + 64 * j];  // the wave's own row: no barrier needed
+}
+
+__global__ void __launch_bounds__(kPlanThreads)
+plan_scan_kernel(uint32_t routes, uint32_t* __restrict__ work, PlanView p, uint32_t gpc) {
+    __shared__ uint32_t part[4][256], cnt[256], rbase[257], gbase[257], cbase[257];
+    const uint32_t tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+    const uint32_t waves = wide_plan_groups(routes) * kPlanWaves;
+    const uint32_t first_bad = work[0];
+    if (first_bad != 0xffffffffu) {
+        __syncthreads();
+        if (tid == 0) {
+            p.meta[kPlanFault] = (first_bad & 15u) == 2 ? 8u : 7u;  // Status::nonfinite : Status::metadata
+            p.meta[kGroupCount] = 0;
+            p.meta[kChunkCount] = 0;
+            work[0] = 0xffffffffu;
+        }
+        return;
+    }
+    // Four threads per expert each total a quarter of the waves, then turn the counts of their
+    // quarter into running starts.
+    uint32_t* counts = work + 4;
+    const uint32_t e = tid & 255, quarter = tid >> 8, per = (waves + 3) / 4;
+    const uint32_t k0 = quarter * per, k1 = k0 + per < waves ? k0 + per : waves;
+    uint32_t sum = 0;
+    for (uint32_t k = k0; k < k1; ++k) sum += counts[uint64_t(k) * 256 + e];
+    part[quarter][e] = sum;
+    __syncthreads();
+    uint32_t run = 0;
+    for (uint32_t qd = 0; qd < quarter; ++qd) run += part[qd][e];
+    if (quarter == 3) cnt[e] = run + sum;
+    for (uint32_t k = k0; k < k1; ++k) {
+        const uint32_t c = counts[uint64_t(k) * 256 + e];
+        counts[uint64_t(k) * 256 + e] = run;
+        run += c;
+    }
+    __syncthreads();
+    if (wv == 0) {
+        uint32_t a[4], b[4], c[4];
+#pragma unroll
+        for (uint32_t j = 0; j < 4; ++j) {
+            a[j] = cnt[4 * lane + j];
+            b[j] = (a[j] + 15) / 16;
+            c[j] = (b[j] + gpc - 1) / gpc;
+        }
+        wave_scan256(a, rbase, lane);
+        wave_scan256(b, gbase, lane);
+        wave_scan256(c, cbase, lane);
+    }
+    __syncthreads();
+    uint32_t* bases = work + 4 + uint64_t(waves) * 256;
+    for (uint32_t i = tid; i < 257; i += kPlanThreads) {
+        bases[i] = rbase[i];
+        bases[257 + i] = gbase[i];
+    }
+    const uint32_t ngroups = gbase[256], nchunks = cbase[256];
+    for (uint32_t gi = tid; gi < ngroups; gi += kPlanThreads) {
+        const uint32_t ex = last_not_above(gbase, gi), k = gi - gbase[ex];
+        const uint32_t left = cnt[ex] - 16 * k, n = left < 16 ? left : 16;
+        Group& G = p.groups[gi];
+        G.expert = int32_t(ex);
+        G.rows = int32_t(n);
+        G.route_base = int32_t(rbase[ex] + 16 * k);
+        for (uint32_t slot = n; slot < 16; ++slot) G.input_rows[slot] = -1;
+    }
+    for (uint32_t ci = tid; ci < nchunks; ci += kPlanThreads) {
+        const uint32_t ex = last_not_above(cbase, ci), j = ci - cbase[ex];
+        const uint32_t ng = (cnt[ex] + 15) / 16, left = ng - gpc * j;
+        p.chunks[ci] = Chunk{int32_t(gbase[ex] + gpc * j), int32_t(left < gpc ? left : gpc)};
+    }
+    if (tid == 0) {
+        p.meta[kGroupCount] = ngroups;
+        p.meta[kChunkCount] = nchunks;
+        p.meta[kPlanFault] = 0;
+    }
+}
+
+__global__ void __launch_bounds__(kPlanThreads)
+plan_place_kernel(const int32_t* __restrict__ ids, const float* __restrict__ w, uint32_t rows,
+                  const uint32_t* __restrict__ work, PlanView p, bool want_gw) {
+    __shared__ uint32_t start[kPlanWaves][256], rbase[257], gbase[257];
+    if (p.meta[kPlanFault]) return;  // a rejected plan writes nothing
+    const uint32_t tid = threadIdx.x, lane = tid & 63, wv = tid >> 6, routes = rows * kTopk;
+    const uint32_t waves = wide_plan_groups(routes) * kPlanWaves;
+    const uint32_t* mine = work + 4 + (uint64_t(blockIdx.x) * kPlanWaves + wv) * 256;
+    const uint32_t* bases = work + 4 + uint64_t(waves) * 256;
+#pragma unroll
+    for (uint32_t j = 0; j < 4; ++j) start[wv][lane + 64 * j] = mine[lane + 64 * j];
+    for (uint32_t i = tid; i < 257; i += kPlanThreads) {
+        rbase[i] = bases[i];
+        gbase[i] = bases[257 + i];
+    }
+    __syncthreads();
+    const uint32_t first_route = blockIdx.x * kWideRoutesPerGroup + wv * kWideRoutesPerWave;
+    int32_t e4[kWideRoutesPerWave / 64];
+    float w4[kWideRoutesPerWave / 64];
+#pragma unroll
+    for (uint32_t step = 0; step < kWideRoutesPerWave / 64; ++step) {  // all loads first: the walk is short
+        const uint32_t i = first_route + step * 64 + lane;
+        e4[step] = i < routes ? ids[i] : 0;
+        w4[step] = i < routes && want_gw ? w[i] : 0.0f;
+    }
+#pragma unroll
+    for (uint32_t step = 0; step < kWideRoutesPerWave / 64; ++step) {
+        const uint32_t i = first_route + step * 64 + lane;
+        const bool valid = i < routes;
+        const uint32_t e = uint32_t(e4[step]) & 255u;
+        const uint64_t m = same_expert_lanes(e, valid);
+        const uint64_t below = m & ((1ull << lane) - 1);
+        if (valid) {
+            const uint32_t rel = start[wv][e] + __popcll(below);
+            const uint32_t pos = rbase[e] + rel;
+            p.original[pos] = int32_t(i);
+            p.inverse[i] = int32_t(pos);
+            p.groups[gbase[e] + rel / 16].input_rows[rel % 16] = int32_t(i / kTopk);
+            if (want_gw) p.gw[pos] = w4[step];
+            if (!below) start[wv][e] += __popcll(m);
+        }
+    }
+}
+
 // Clears the per-call stage fault words; runs ahead of the planner on the same stream.
 __global__ void meta_reset_kernel(uint32_t* meta) {
     if (threadIdx.x < kMetaWords) meta[threadIdx.x] = threadIdx.x == kQuantWhere ? 0xffffffffu : 0u;

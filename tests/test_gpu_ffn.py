@@ -193,6 +193,10 @@ def test_prefill_chunk_properties_and_sampled_parity(full_layer):
     n = wl.rows * 8
     orig, inv = s.view("original_routes", np.int32, n), s.view("inverse", np.int32, n)
     assert np.array_equal(np.sort(orig), np.arange(n)) and np.array_equal(inv[orig], np.arange(n))
+    ref = O.plan(8192, wl.ids, wl.weights)                                 # the planner spread over several compute units
+    assert ref.status == 0 and stats.groups == int(ref.group_count[0])
+    assert np.array_equal(orig, ref.original_routes[:n]) and np.array_equal(inv, ref.inverse[:n])
+    assert np.array_equal(s.view("groups", O.GROUP_DTYPE, stats.groups), ref.groups[:stats.groups])
     experts = wl.ids.reshape(-1)[orig]
     assert np.all(np.diff(experts) >= 0)
     same = np.diff(experts) == 0
@@ -242,6 +246,37 @@ def test_errors_and_faults(full_layer):
     assert lib.m26s_b1_layer_new(1, 5, 0, C.byref(C.c_void_p()), buf, 256) == 1 and b"bad canonical extent/rank" in buf.value
     st = b1.ffn(layer, s, wl.payload, wl.scales, wl.ids, wl.weights, wl.rows, out)   # the scratch recovers after faults
     assert st.groups > 0 and out.any()
+
+
+def test_wide_planner_faults_and_recovery(full_layer):
+    """Above 512 rows the planner runs as three launches over several compute units: the same faults in
+    the same order of precedence, nothing written by a rejected plan, and the next call is clean."""
+    _, pools, layer = full_layer
+    wl = synth.make(3, rows=1536)
+    s = b1.Scratch()
+    s.set_taps(True)                                                     # also fills grouped_weights
+    out = np.zeros((wl.rows, 4096), np.uint16)
+    n = wl.rows * 8
+    b1.ffn(layer, s, wl.payload, wl.scales, wl.ids, wl.weights, wl.rows, out)
+    ref = O.plan(2048, wl.ids, wl.weights)
+    good = [s.view(k, np.int32, n).copy() for k in ("original_routes", "inverse")]
+    assert np.array_equal(good[0], ref.original_routes[:n]) and np.array_equal(good[1], ref.inverse[:n])
+    assert np.array_equal(s.view("grouped_weights", np.float32, n), ref.grouped_weights[:n])
+    cases = []
+    ids = wl.ids.copy(); ids[1400, 7] = ids[1400, 0]; cases.append((ids, wl.weights))          # repeat inside a token
+    ids = wl.ids.copy(); ids[700, 2] = 256; cases.append((ids, wl.weights))                     # id out of range
+    ids = wl.ids.copy(); ids[3, 1] = -1; cases.append((ids, wl.weights))
+    w = wl.weights.copy(); w[1535, 7] = -1.0; cases.append((wl.ids, w))                         # negative weight
+    w = wl.weights.copy(); w[600, 0] = np.inf; cases.append((wl.ids, w))
+    for bad_ids, bad_w in cases:
+        with pytest.raises(b1.B1Error, match="invalid routes") as e:
+            b1.ffn(layer, s, wl.payload, wl.scales, bad_ids, bad_w, wl.rows, out)
+        assert e.value.code == 3
+        assert np.array_equal(s.view("original_routes", np.int32, n), good[0])   # the rejected plan wrote nothing
+        assert np.array_equal(s.view("inverse", np.int32, n), good[1])
+    out2 = np.zeros_like(out)
+    st = b1.ffn(layer, s, wl.payload, wl.scales, wl.ids, wl.weights, wl.rows, out2)
+    assert st.groups == int(ref.group_count[0]) and np.array_equal(out2, out)
 
 
 def test_abnormal_weight_scales_are_refused():
