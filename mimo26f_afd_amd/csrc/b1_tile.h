@@ -386,7 +386,31 @@ __device__ __forceinline__ void fc2_tile_body(const Fc2Args& a, const Chunk ch, 
         const bool live = tt < ch.groups && int32_t(r2) < grp[tt].rows;
         route[tt] = live ? a.plan.original[grp[tt].route_base + r2] : -1;
     }
-    fc2_finish<TT>(a, ob, lane2, acc, route);
+    // A lane holds four consecutive output columns of one token per tile, so a store straight from the
+    // accumulators touches sixteen token rows with 64 bytes each. One trip through the wave's own, now
+    // idle, weight ring regroups a tile row into 256 contiguous bytes per token (sixteen lanes) and
+    // four tokens per store: a tenth off the kernel at 8192 tokens. Cells are 272 bytes apart so the
+    // regrouped reads (same token, sixteen cells) fall on different banks.
+    uint8_t* ring = lds + wv * (kWeightStages * 4096);
+    const uint32_t cell = lane2 & 15, token4 = lane2 >> 4;  // regrouped: sixteen 16-byte cells of one token, four tokens
+    const uint32_t put_at = uint32_t(uintptr_t((lds_ptr)ring)) + (lane2 >> 4) * 272 + (lane2 & 15) * 16;
+    bool lost = false;
+#pragma unroll
+    for (int tt = 0; tt < TT; ++tt) {
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+            asm volatile("ds_write_b128 %0, %1 offset:%2" ::"v"(put_at), "a"(acc[t][tt]), "n"(t * 4 * 272) : "memory");
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const uint32_t token = 4 * j + token4;
+            const v4f v = *reinterpret_cast<const v4f*>(ring + cell * 272 + token * 16);
+            const int32_t rt = __shfl(route[tt], int(token));
+            if (rt < 0) continue;
+            if (uint32_t(rt) >= a.routes) { lost = true; continue; }
+            *reinterpret_cast<v4f*>(a.y + size_t(rt) * kHidden + ob * 64 + cell * 4) = v;
+        }
+    }
+    if (lost) atomicOr(&a.plan.meta[kFc2Fault], 5u);
 }
 
 // Work item of a tile workgroup. Workgroups are handed to the eight XCDs in turn, each with an L2 of
