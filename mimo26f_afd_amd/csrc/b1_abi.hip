@@ -84,7 +84,7 @@ struct m26s_b1_scratch {
     hipStream_t st = nullptr;
     bool own_stream = false;
     hipEvent_t e0 = nullptr, ep = nullptr, ea = nullptr, ec = nullptr, e1 = nullptr;
-    Dev x, xs, iw, inv, orig, gw, groups, chunks, meta, dq, dqs, y, bf16, pad, tap_gate, tap_up, tap_h, xg, rowbad, dg, planw;
+    Dev x, xs, iw, inv, orig, gw, groups, chunks, meta, dq, dqs, y, bf16, pad, tap_gate, tap_up, tap_h, xg, rowbad, dg, planw, xrows, yrows;
     std::vector<uint8_t> hiw;
     bool taps = false;
     uint32_t last_rows = 0, last_inter = 0;
@@ -159,11 +159,11 @@ void launch_ffn(const m26s_b1_layer* L, m26s_b1_scratch* S, const PlanView& pv, 
     const uint8_t* zero = S->pad.as<uint8_t>();
     Fc1Args f1{L->prepared, L->lay, pv, x, xp, xs, xsp, zero, zero + 8192, S->dq.as<uint8_t>(), S->dqs.as<uint8_t>(),
                S->taps ? S->tap_gate.as<float>() : nullptr, S->taps ? S->tap_up.as<float>() : nullptr,
-               S->taps ? S->tap_h.as<float>() : nullptr, nullptr, nullptr, nullptr};
+               S->taps ? S->tap_h.as<float>() : nullptr, nullptr, nullptr, nullptr, nullptr};
     fc1_kernel<NT><<<dim3(L->lay.inter / 128, chunk_cap), 256, 0, S->st>>>(f1);
     (void)hipEventRecord(S->ea, S->st);
     Fc2Args f2{L->prepared, L->lay, pv, S->dq.as<uint8_t>(), S->dqs.as<uint8_t>(), zero, zero + 8192,
-               S->y.as<float>(), uint32_t(routes), nullptr};
+               S->y.as<float>(), uint32_t(routes), nullptr, nullptr, nullptr};
     fc2_kernel<NT><<<dim3(16, chunk_cap), 256, 0, S->st>>>(f2);
     (void)hipEventRecord(S->ec, S->st);
 }
@@ -173,14 +173,16 @@ void launch_tiles(const m26s_b1_layer* L, m26s_b1_scratch* S, const PlanView& pv
                   const uint8_t* xs, size_t xsp, uint32_t chunk_cap, uint64_t routes) {
     const uint8_t* zero = S->pad.as<uint8_t>();
     const uint32_t inter = L->lay.inter;
-    gather_scales_kernel<<<chunk_cap, 256, 0, S->st>>>(pv, xs, xsp, S->xg.as<uint32_t>(), S->rowbad.as<uint32_t>());
+    gather_scales_kernel<<<chunk_cap, 256, 0, S->st>>>(pv, xs, xsp, S->xg.as<uint32_t>(), S->rowbad.as<uint32_t>(),
+                                                     S->xrows.as<int32_t>(), S->yrows.as<int32_t>());
     Fc1Args f1{L->prepared, L->lay, pv, x, xp, xs, xsp, zero, zero + 8192, S->dq.as<uint8_t>(), S->dqs.as<uint8_t>(),
                S->taps ? S->tap_gate.as<float>() : nullptr, S->taps ? S->tap_up.as<float>() : nullptr,
-               S->taps ? S->tap_h.as<float>() : nullptr, S->xg.as<uint8_t>(), S->rowbad.as<uint32_t>(), S->dg.as<uint8_t>()};
+               S->taps ? S->tap_h.as<float>() : nullptr, S->xg.as<uint8_t>(), S->rowbad.as<uint32_t>(), S->xrows.as<int32_t>(),
+               S->dg.as<uint8_t>()};
     fc1_tile_kernel<<<tile_grid(inter / 128, chunk_cap), kTileThreads, kTileLdsBytes, S->st>>>(f1);
     (void)hipEventRecord(S->ea, S->st);
     Fc2Args f2{L->prepared, L->lay, pv, S->dq.as<uint8_t>(), S->dqs.as<uint8_t>(), zero, zero + 8192,
-               S->y.as<float>(), uint32_t(routes), S->dg.as<uint8_t>()};
+               S->y.as<float>(), uint32_t(routes), S->dg.as<uint8_t>(), S->yrows.as<int32_t>(), S->rowbad.as<uint32_t>()};
     fc2_tile_kernel<<<tile_grid(kHidden / 256, chunk_cap), kTileThreads, kTileLdsBytes, S->st>>>(f2);
     (void)hipEventRecord(S->ec, S->st);
 }
@@ -205,6 +207,8 @@ int enqueue(const m26s_b1_layer* L, m26s_b1_scratch* S, const uint8_t* x, size_t
         M26S_CK(S->xg.ensure(ccap * gathered_scale_bytes(kHidden)), "b1 gathered input scales alloc");
         M26S_CK(S->dg.ensure(ccap * gathered_scale_bytes(inter)), "b1 gathered intermediate scales alloc");
         M26S_CK(S->rowbad.ensure(ccap * 16 * 4), "b1 row verdict alloc");
+        M26S_CK(S->xrows.ensure(ccap * 128 * 4), "b1 chunk row table alloc");
+        M26S_CK(S->yrows.ensure(ccap * 128 * 4), "b1 chunk route table alloc");
     }
     if (S->taps) {
         M26S_CK(S->tap_gate.ensure(gcap * 16 * inter * 4), "b1 gate tap alloc");

@@ -291,7 +291,7 @@ plan_kernel(const int32_t* __restrict__ ids, const float* __restrict__ w, uint32
     for (uint32_t ci = tid; ci < nchunks; ci += kPlanThreads) {
         const uint32_t e = last_not_above(cbase, ci), j = ci - cbase[e];
         const uint32_t ng = (cnt[e] + 15) / 16, left = ng - gpc * j;
-        p.chunks[ci] = Chunk{int32_t(gbase[e] + gpc * j), int32_t(left < gpc ? left : gpc)};
+        p.chunks[ci] = Chunk{int32_t(gbase[e] + gpc * j), int32_t(left < gpc ? left : gpc), int32_t(e), 0};
     }
     if (tid == 0) {
         p.meta[kGroupCount] = ngroups;
@@ -440,7 +440,7 @@ plan_scan_kernel(uint32_t routes, uint32_t* __restrict__ work, PlanView p, uint3
     for (uint32_t ci = tid; ci < nchunks; ci += kPlanThreads) {
         const uint32_t ex = last_not_above(cbase, ci), j = ci - cbase[ex];
         const uint32_t ng = (cnt[ex] + 15) / 16, left = ng - gpc * j;
-        p.chunks[ci] = Chunk{int32_t(gbase[ex] + gpc * j), int32_t(left < gpc ? left : gpc)};
+        p.chunks[ci] = Chunk{int32_t(gbase[ex] + gpc * j), int32_t(left < gpc ? left : gpc), int32_t(ex), 0};
     }
     if (tid == 0) {
         p.meta[kGroupCount] = ngroups;
@@ -696,6 +696,7 @@ struct Fc1Args {
     const uint8_t* xg;     // FC1 input scales, gathered by gather_scales_kernel
     const uint32_t* rowbad;  // [chunk][16]: bit 0 set where a row index of the chunk met an illegal input scale,
                              // bit 8+t set where tile t holds a token in that row
+    const int32_t* xrows;    // [chunk][8 tiles][16]: the token each row of each tile reads, -1 for none
     uint8_t* dg;           // the intermediate's scales in the same order, written here for FC2
 };
 
@@ -788,7 +789,7 @@ template <int TT>
 __device__ __forceinline__ void fc1_body(const Fc1Args& a, const Chunk ch, uint32_t cb, uint32_t lane) {
     const uint32_t r = lane & 15, g = lane >> 4;
     const Group* grp = a.plan.groups + ch.first_group;
-    const int32_t expert = grp[0].expert;
+    const int32_t expert = ch.expert;
     const uint8_t* xrow[TT];
     const uint8_t* xsrow[TT];
     bool live[TT];
@@ -823,7 +824,7 @@ __global__ void __launch_bounds__(256) fc1_kernel(Fc1Args a) {
     if (meta[kPlanFault] || c >= meta[kChunkCount]) return;
     const Chunk ch = a.plan.chunks[c];
     const uint32_t lane = threadIdx.x & 63, cb = blockIdx.x * 4 + (threadIdx.x >> 6);
-    const int32_t expert = a.plan.groups[ch.first_group].expert;
+    const int32_t expert = ch.expert;
     if (expert < 0 || expert >= int32_t(kExperts) || ch.groups < 1 || ch.groups > NT) {
         if (lane == 0) atomicOr(&meta[kFc1Fault], 2u);
         return;
@@ -845,6 +846,8 @@ struct Fc2Args {
     float* y;         // [routes][4096], original (token, slot) order, unweighted
     uint32_t routes;
     const uint8_t* dg;  // tile schedule only: the intermediate's scales in MFMA lane order (see Fc1Args)
+    const int32_t* yrows;  // tile schedule only, [chunk][8 tiles][16]: the route (row of y) of each row, -1 for none
+    const uint32_t* rowbad;  // tile schedule only: as in Fc1Args (bit 8+t: tile t holds a token in that row)
 };
 
 // FC2 epilogue of one wave: unweighted FP32 rows back to y[original route].
@@ -869,7 +872,7 @@ template <int TT>
 __device__ __forceinline__ void fc2_body(const Fc2Args& a, const Chunk ch, uint32_t ob, uint32_t lane) {
     const uint32_t r = lane & 15, g = lane >> 4, I = a.lay.inter;
     const Group* grp = a.plan.groups + ch.first_group;
-    const int32_t expert = grp[0].expert;
+    const int32_t expert = ch.expert;
     const uint8_t* xrow[TT];
     const uint8_t* xsrow[TT];
     int32_t route[TT];
@@ -904,7 +907,7 @@ __global__ void __launch_bounds__(256) fc2_kernel(Fc2Args a) {
     if (meta[kPlanFault] || meta[kFc1Fault] || meta[kQuantFault] || c >= meta[kChunkCount]) return;
     const Chunk ch = a.plan.chunks[c];
     const uint32_t lane = threadIdx.x & 63, ob = blockIdx.x * 4 + (threadIdx.x >> 6);
-    const int32_t expert = a.plan.groups[ch.first_group].expert;
+    const int32_t expert = ch.expert;
     if (expert < 0 || expert >= int32_t(kExperts) || ch.groups < 1 || ch.groups > NT) {
         if (lane == 0) atomicOr(&meta[kFc2Fault], 2u);
         return;

@@ -53,7 +53,10 @@ struct Group {
 static_assert(sizeof(Group) == 76, "Group is 19 int32");
 struct Chunk {
     int32_t first_group, groups;
+    int32_t expert;    // the groups' expert, so a kernel can address the weights one load after its index
+    int32_t reserved;  // zero
 };
+static_assert(sizeof(Chunk) == 16, "Chunk is four int32");
 
 // meta words written by the planner and the stage kernels; one small device array per scratch.
 enum Meta : uint32_t {

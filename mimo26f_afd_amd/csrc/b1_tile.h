@@ -81,10 +81,12 @@ __device__ __forceinline__ void mfma_acc(v4f& acc, const v4i& a, const v8i& b, u
 // checks them against the legal window [105, 247] (crates/mimo26-expert/kernels/b1/grouped.cu:28,37
 // holds the reference's check). Padded rows get the unit scale 127. rowbad[chunk][r] collects, for
 // row r of all tiles, the verdict in bit 0 (the granularity the FC1 epilogue reports faults at) and
-// in bit 8+t whether tile t holds a token there, so the epilogue looks nothing else up.
+// in bit 8+t whether tile t holds a token there, so the epilogue looks nothing else up. xrows / yrows
+// list, per tile and row, the token FC1 reads and the route FC2 writes (-1 for none).
 // grid (chunk capacity), 256 threads = 8 tiles x 16 rows x 2 halves of a scale row.
 __global__ void __launch_bounds__(256) gather_scales_kernel(PlanView plan, const uint8_t* __restrict__ xs, size_t xs_pitch,
-                                                            uint32_t* __restrict__ xg, uint32_t* __restrict__ rowbad) {
+                                                            uint32_t* __restrict__ xg, uint32_t* __restrict__ rowbad,
+                                                            int32_t* __restrict__ xrows, int32_t* __restrict__ yrows) {
     __shared__ uint32_t flags[16];
     const uint32_t c = blockIdx.x, tid = threadIdx.x;
     if (plan.meta[kPlanFault] || c >= plan.meta[kChunkCount]) return;
@@ -94,6 +96,10 @@ __global__ void __launch_bounds__(256) gather_scales_kernel(PlanView plan, const
     if (tid < 16) flags[tid] = 0;
     __syncthreads();
     const int32_t row = int32_t(tt) < ch.groups ? plan.groups[ch.first_group + tt].input_rows[r] : -1;
+    if (half == 0) {  // the chunk's rows flattened: FC1 and FC2 find them one load after their chunk index
+        xrows[c * 128 + tt * 16 + r] = row;
+        yrows[c * 128 + tt * 16 + r] = row >= 0 ? plan.original[plan.groups[ch.first_group + tt].route_base + r] : -1;
+    }
     uint32_t bad = 0;
 #pragma unroll
     for (uint32_t j = 0; j < 4; ++j) {
@@ -299,13 +305,12 @@ __device__ __forceinline__ void fc1_tile_body(const Fc1Args& a, const Chunk ch, 
                                               uint32_t lane, uint8_t* lds) {
     constexpr int kMine = TT / kTileWaves;
     const uint32_t r = lane & 15, g = lane >> 4;
-    const Group* grp = a.plan.groups + ch.first_group;
-    const int32_t expert = grp[0].expert;
+    const int32_t expert = ch.expert;
     const uint8_t* row[kMine];
 #pragma unroll
     for (int m = 0; m < kMine; ++m) {
         const int lt = int(wv) * kMine + m;
-        const int32_t mine = lt < ch.groups ? grp[lt].input_rows[r] : -1;
+        const int32_t mine = a.xrows[c * 128 + lt * 16 + r];
         row[m] = (mine >= 0 ? a.x + size_t(mine) * a.x_pitch : a.zero_row) + g * 16;
     }
     const uint8_t* img = a.prepared + uint64_t(expert) * a.lay.bytes();
@@ -358,13 +363,13 @@ __device__ __forceinline__ void fc2_tile_body(const Fc2Args& a, const Chunk ch, 
                                               uint32_t lane, uint8_t* lds) {
     constexpr int kMine = TT / kTileWaves;
     const uint32_t r = lane & 15, g = lane >> 4, I = a.lay.inter;
-    const Group* grp = a.plan.groups + ch.first_group;
-    const int32_t expert = grp[0].expert;
+    const int32_t expert = ch.expert;
+    const uint32_t verdict = a.rowbad[c * 16 + r];  // bit 8+t: tile t holds a token in this row
     const uint8_t* row[kMine];
 #pragma unroll
     for (int m = 0; m < kMine; ++m) {
         const int lt = int(wv) * kMine + m;
-        const bool mine = lt < ch.groups && int32_t(r) < grp[lt].rows;
+        const bool mine = (verdict >> (8 + lt)) & 1u;
         const size_t grow = size_t(ch.first_group + lt) * 16 + r;
         row[m] = (mine ? a.dq + grow * I : a.zero_row) + g * 16;
     }
@@ -379,13 +384,7 @@ __device__ __forceinline__ void fc2_tile_body(const Fc2Args& a, const Chunk ch, 
 #pragma unroll
         for (int tt = 0; tt < TT; ++tt) acc[t][tt] = v4f{0.f, 0.f, 0.f, 0.f};
     gemm_chunk_lds<TT>(acc, wp, sp, sx, int(ksteps), row, wv, lane, lds);
-    const uint32_t lane2 = after_loop(lane), r2 = lane2 & 15;
-    int32_t route[TT];
-#pragma unroll
-    for (int tt = 0; tt < TT; ++tt) {
-        const bool live = tt < ch.groups && int32_t(r2) < grp[tt].rows;
-        route[tt] = live ? a.plan.original[grp[tt].route_base + r2] : -1;
-    }
+    const uint32_t lane2 = after_loop(lane);
     // A lane holds four consecutive output columns of one token per tile, so a store straight from the
     // accumulators touches sixteen token rows with 64 bytes each. One trip through the wave's own, now
     // idle, weight ring regroups a tile row into 256 contiguous bytes per token (sixteen lanes) and
@@ -395,6 +394,11 @@ __device__ __forceinline__ void fc2_tile_body(const Fc2Args& a, const Chunk ch, 
     const uint32_t cell = lane2 & 15, token4 = lane2 >> 4;  // regrouped: sixteen 16-byte cells of one token, four tokens
     const uint32_t put_at = uint32_t(uintptr_t((lds_ptr)ring)) + (lane2 >> 4) * 272 + (lane2 & 15) * 16;
     bool lost = false;
+    int32_t route[TT][4];  // all looked up at once: one latency, not thirty-two
+#pragma unroll
+    for (int tt = 0; tt < TT; ++tt)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) route[tt][j] = a.yrows[c * 128 + tt * 16 + 4 * j + token4];
 #pragma unroll
     for (int tt = 0; tt < TT; ++tt) {
 #pragma unroll
@@ -404,7 +408,7 @@ __device__ __forceinline__ void fc2_tile_body(const Fc2Args& a, const Chunk ch, 
         for (int j = 0; j < 4; ++j) {
             const uint32_t token = 4 * j + token4;
             const v4f v = *reinterpret_cast<const v4f*>(ring + cell * 272 + token * 16);
-            const int32_t rt = __shfl(route[tt], int(token));
+            const int32_t rt = route[tt][j];
             if (rt < 0) continue;
             if (uint32_t(rt) >= a.routes) { lost = true; continue; }
             *reinterpret_cast<v4f*>(a.y + size_t(rt) * kHidden + ob * 64 + cell * 4) = v;
@@ -434,7 +438,7 @@ __global__ void __launch_bounds__(kTileThreads, 2) fc1_tile_kernel(Fc1Args a) {
     if (meta[kPlanFault] || c >= meta[kChunkCount]) return;
     const Chunk ch = a.plan.chunks[c];
     const uint32_t lane = threadIdx.x & 63, wv = threadIdx.x >> 6, cb = it.column * 4 + wv;
-    const int32_t expert = a.plan.groups[ch.first_group].expert;
+    const int32_t expert = ch.expert;
     if (expert < 0 || expert >= int32_t(kExperts) || ch.groups < 1 || ch.groups > 8) {
         if (lane == 0) atomicOr(&meta[kFc1Fault], 2u);
         return;
@@ -454,7 +458,7 @@ __global__ void __launch_bounds__(kTileThreads, 2) fc2_tile_kernel(Fc2Args a) {
     if (meta[kPlanFault] || meta[kFc1Fault] || meta[kQuantFault] || c >= meta[kChunkCount]) return;
     const Chunk ch = a.plan.chunks[c];
     const uint32_t lane = threadIdx.x & 63, wv = threadIdx.x >> 6, ob = it.column * 4 + wv;
-    const int32_t expert = a.plan.groups[ch.first_group].expert;
+    const int32_t expert = ch.expert;
     if (expert < 0 || expert >= int32_t(kExperts) || ch.groups < 1 || ch.groups > 8) {
         if (lane == 0) atomicOr(&meta[kFc2Fault], 2u);
         return;
