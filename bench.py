@@ -132,6 +132,88 @@ def run_config(cfg, steps, warmup, torch, dev, b1, synth, O, parity_tokens, cpu_
     return res
 
 
+def run_stack(args, torch, dev, O):
+    """configs[4]: the routed experts of `--stack` layers resident in HBM; a prefill in 4096-token
+    segments, a 16-token decode step after each; one JSON line of its own."""
+    from mimo26f_afd_amd import stack as S, synth
+    layers, tokens, seg, dec_rows = args.stack, args.stack_tokens, 4096, 16
+    segments = tokens // seg
+    t0 = time.time()
+    st = S.ResidentStack(layers, torch, dev, log=log)
+    log(f"[bench] {layers} layers prepared in {time.time() - t0:.1f}s")
+    pre_routes, dec_routes = st.routes(seg, 0), st.routes(dec_rows, 1)
+    x_pre = S.activations_dev(torch, dev, st.seed, tokens, 0)
+    x_dec = S.activations_dev(torch, dev, st.seed, dec_rows, 1)
+    buf_pre, buf_dec = st.buffers(seg), st.buffers(dec_rows)
+    ev = lambda: torch.cuda.Event(enable_timing=True)
+    check_layers = sorted({0, layers // 2, layers - 1})
+    kept = {}
+
+    def sweep(x, routes, buf, timers, keep_as=None):
+        for l in range(layers):
+            pair = (ev(), ev())
+            nxt = st.layer_step(l, x, routes[l][0], routes[l][1], buf, pair)
+            timers.append(pair)
+            if keep_as is not None and l in check_layers:  # a few rows of this layer's input and output, for the CPU check
+                kept[(keep_as, l)] = (buf["frame"][:8].cpu().numpy(), routes[l][0][:8].cpu().numpy(),
+                                      routes[l][1][:8].cpu().numpy(), buf["out"][:8].view(torch.int16).cpu().numpy().view(np.uint16))
+            x = nxt
+        return x
+
+    # warm-up: one segment and one decode step through every layer, kept for the parity sample
+    last = sweep(x_pre[:seg], pre_routes, buf_pre, [], "prefill")
+    sweep(x_dec, dec_routes, buf_dec, [], "decode")
+    st.sync()
+    torch.cuda.synchronize()
+    pre_t, dec_t = [], []
+    e0, e1 = ev(), ev()
+    t0 = time.perf_counter()
+    e0.record()
+    for sgm in range(segments):
+        last = sweep(x_pre[sgm * seg:(sgm + 1) * seg], pre_routes, buf_pre, pre_t)
+        x_dec = sweep(x_dec, dec_routes, buf_dec, dec_t)
+    e1.record()
+    st.sync()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    pre_ms = np.array([a.elapsed_time(b) for a, b in pre_t])
+    dec_ms = np.array([a.elapsed_time(b) for a, b in dec_t])
+    parity = []
+    for (kind, l), (frame, ids, w, got) in sorted(kept.items()):
+        rc, ref = S.reference_rows(st.seed, l, frame[:, :4096].copy(), frame[:, 4096:4224].copy(), ids, w, O)
+        g = (got.astype(np.uint32) << 16).view(np.float32).astype(np.float64)
+        r = (ref.astype(np.uint32) << 16).view(np.float32).astype(np.float64)
+        parity.append(dict(batch=kind, layer=l, tokens=len(ids), oracle_rc=rc, max_abs_over_max_ref=float(np.max(np.abs(g - r)) / np.max(np.abs(r))),
+                           mean_rel=float(np.sum(np.abs(g - r)) / np.sum(np.abs(r)))))
+    touched = np.mean([np.unique(r[0].cpu().numpy()).size for r in dec_routes])
+    dec_bytes = touched * synth.IMAGE_BYTES * 4 + dec_rows * (4224 + 64 + 8192)
+    flops = 6 * seg * 8 * 4096 * 2048
+    calls = segments * layers
+    line = {
+        "metric": "routed tok/s per MoE layer; HBM GB/s (decode) and MFMA % of peak (prefill)",
+        "value": (seg + dec_rows) * calls / (wall_ms * 1e-3), "unit": "routed tok/s per MoE layer",
+        "n_gpus": 1, "steps": segments, "warmup": 1, "ms_per_step": wall_ms / segments,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "fp8xfp4->f32", "data": "synthetic",
+        "config": {"workload": f"configs[4]: {layers} MoE layers' routed experts resident in HBM ({layers * 256 * synth.IMAGE_BYTES * 4 / 1e9:.1f} GB "
+                               f"canonical), {tokens}-token prefill in {seg}-token segments, a {dec_rows}-token decode step after each; "
+                               "per layer: wire quantizer -> FFN -> residual mix",
+                   "whole_schedule_ms": wall_ms, "event_ms": e0.elapsed_time(e1),
+                   "hbm_held_GiB": (torch.cuda.mem_get_info()[1] - torch.cuda.mem_get_info()[0]) / 2**30,
+                   "final_residual_std": float(last.std())},
+        "prefill_ffn": {"ms_per_layer_call": float(np.median(pre_ms)), "min": float(pre_ms.min()), "max": float(pre_ms.max()),
+                        "tok_per_s": seg / (float(np.median(pre_ms)) * 1e-3),
+                        "tflops": flops / (float(np.median(pre_ms)) * 1e-3) / 1e12,
+                        "frac_of_fp8_peak": flops / (float(np.median(pre_ms)) * 1e-3) / 1e12 / MFMA_FP8_PEAK_TFLOPS},
+        "decode_ffn": {"ms_per_layer_call": float(np.median(dec_ms)), "min": float(dec_ms.min()), "max": float(dec_ms.max()),
+                       "tok_per_s": dec_rows / (float(np.median(dec_ms)) * 1e-3), "experts_touched_mean": float(touched),
+                       "GBps": dec_bytes / (float(np.median(dec_ms)) * 1e-3) / 1e9,
+                       "frac_of_hbm_peak": dec_bytes / (float(np.median(dec_ms)) * 1e-3) / 1e9 / HBM_PEAK_GBS},
+        "parity": parity,
+    }
+    st.close()
+    print(json.dumps(line), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -144,6 +226,9 @@ def main():
                          "size that scales the FETCH_SIZE / WRITE_SIZE counters")
     ap.add_argument("--only-prefill", action="store_true",
                     help="profiling aid: run only the prefill measurement and print its object")
+    ap.add_argument("--stack", type=int, default=0, metavar="LAYERS",
+                    help="run configs[4] instead: this many layers' routed experts resident in HBM (48 = the full model, 164 GB)")
+    ap.add_argument("--stack-tokens", type=int, default=65536, help="prefill length of the --stack run (a multiple of 4096)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU only (no collectives, no sharding); use --gpus 1")
@@ -156,6 +241,9 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
 
+    if args.stack:
+        run_stack(args, torch, dev, O)
+        return
     if args.copy_probe:
         src = torch.zeros(1 << 28, dtype=torch.int32, device=dev)
         dst = torch.empty_like(src)

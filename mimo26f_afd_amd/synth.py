@@ -67,9 +67,9 @@ def bf16_round(x: np.ndarray) -> np.ndarray:
 
 
 # ---- weights ---------------------------------------------------------------------------------
-def expert_image(seed: int, rank: int, expert: int) -> np.ndarray:
-    """One quarter-slice image v2 (3,342,336 bytes) of `expert` for TP4 rank `rank`."""
-    raw = u64(stream_key(seed, WEIGHTS, rank, expert), IMAGE_BYTES // 8).view(np.uint8).copy()
+def expert_image(seed: int, rank: int, expert: int, layer: int = 0) -> np.ndarray:
+    """One quarter-slice image v2 (3,342,336 bytes) of `expert` of `layer` for TP4 rank `rank`."""
+    raw = u64(stream_key(seed, WEIGHTS, rank, layer * EXPERTS + expert), IMAGE_BYTES // 8).view(np.uint8).copy()
     for lo, hi in SCALE_REGIONS:
         raw[lo:hi] = 119 + ((raw[lo:hi].astype(np.uint16) * 5) >> 8).astype(np.uint8)
     return raw
