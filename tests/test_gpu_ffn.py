@@ -164,6 +164,33 @@ def test_tile_schedule_at_rank_share_stage_by_stage(scratch):
     check_stages(scratch, layer, wl, pools, stats, experts=12)
 
 
+def _skewed_routes(seed, rows, experts):
+    """8 distinct experts per token out of `experts`, Zipf(1.1) popularity (exponential-key sampling)."""
+    p = 1.0 / np.arange(1, len(experts) + 1, dtype=np.float64) ** 1.1
+    u = synth.uniform(synth.stream_key(seed, synth.ROUTES, 5), rows * len(experts)).reshape(rows, len(experts))
+    ranks = np.argsort(-np.log(u) / p, axis=1, kind="stable")[:, :8]
+    return np.asarray(experts, np.int32)[ranks]
+
+
+def test_ragged_sizes_across_the_schedules(scratch):
+    """Row counts either side of every switch of schedule (one and two activation tiles per wave up to
+    32 and 128 rows, the tile kernels above, the planner over several compute units above 512) with
+    skewed routing, so chunks are ragged: plan bit-exact, stages and outputs to the bars."""
+    seed = synth.BASE_SEED + 11
+    experts = list(range(3, 256, 11))  # 23 experts
+    pools = [synth.rank_pool(seed, 0, experts)]
+    layer = DeviceLayer(pools).layer
+    for rows in (1, 31, 33, 127, 129, 130, 191, 513):
+        ids, w, x = _skewed_routes(seed + rows, rows, experts), synth._softmax_weights(seed + rows, rows), synth._activations(seed + rows, rows)
+        payload, scales = synth.q0_quantize(x)
+        wl = synth.Workload(f"ragged {rows}", 1, seed, 1, rows, ids, w, x, payload, scales)
+        stats, bf, pf = run_ffn_dev(layer, scratch, wl)
+        rc, ref_partial, ref_bf16, _ = O.layer_ffn(pools, wl.payload, wl.scales, wl.ids, wl.weights)
+        assert rc == 0, rows
+        check_outputs(pf, bf, ref_partial, ref_bf16)
+        check_stages(scratch, layer, wl, pools, stats, experts=2)
+
+
 @pytest.fixture(scope="module")
 def full_layer():
     wl = synth.make(2)
