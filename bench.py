@@ -285,6 +285,13 @@ def main():
         "cpu_baseline": dec["cpu"],
         "parity": dec["parity"],
     }
+    # The same figures against what this box sustains: a streaming read of 4 GiB, and the GEMMs' MFMA alone.
+    from mimo26f_afd_amd import probe
+    read_gbs = probe.read_bandwidth_gbps()
+    line["roofline"]["measured_read_GBps"] = read_gbs
+    line["roofline"]["frac_of_measured"] = fc1_gbs / read_gbs
+    line["roofline"]["path"]["frac_of_measured"] = path_gbs / read_gbs
+    line["value_routes_per_s"] = line["value"] * 8
     if not args.no_prefill:
         pre = run_config(3, max(3, args.steps // 5), max(2, args.warmup // 5), torch, dev, b1, synth, O, parity_tokens=4,
                          cpu_tokens=0)
@@ -305,6 +312,10 @@ def main():
                                   "reduce_ms": pre["phases"]["reduce_ms"]}},
             "parity": pre["parity"],
         }
+        mfma_tf = probe.mfma_rate_tflops()
+        line["prefill"]["roofline"]["measured_mfma_TFLOPs"] = mfma_tf
+        line["prefill"]["roofline"]["frac_of_measured"] = fc1_tf / mfma_tf
+        line["prefill"]["roofline"]["path"]["frac_of_measured"] = tf / mfma_tf
     print(json.dumps(line), flush=True)
 
 

@@ -150,3 +150,17 @@ def test_chain_router_quantizer_frame_ffn():
     out2, dp, ds = D(wl.rows * 4096 * 2), dev(ref_p), dev(ref_s)  # the same call on the checker's bytes, separate arrays
     b1.ffn_dev(layer, scratch, dp.ptr, 4096, ds.ptr, 128, di.ptr, dw.ptr, wl.rows, out2.ptr)
     assert np.array_equal(out2.to_host(np.uint16).reshape(wl.rows, 4096), got)
+
+
+def test_roofline_probes_report_plausible_rates():
+    """The two measurement aids: a streaming read lands between a third of the HBM peak and the peak,
+    the MFMA-only loop between a third of the FP8 peak and the peak; bad arguments are refused."""
+    from mimo26f_afd_amd import probe
+    gbs = probe.read_bandwidth_gbps(1 << 30, 3)
+    assert 2600 < gbs < 8000, gbs
+    tf = probe.mfma_rate_tflops(500, 2)
+    assert 1600 < tf < 5000, tf
+    with pytest.raises(probe.ProbeError):
+        probe.read_bandwidth_gbps(12345, 1)
+    with pytest.raises(probe.ProbeError):
+        probe.mfma_rate_tflops(0, 1)
