@@ -62,6 +62,17 @@ int m26s_b1_layer_new_full(const uint8_t* const rank_images_dev[4], uint64_t byt
 /* Intermediate columns the layer holds: 512 (one rank) or 2048 (full). */
 uint32_t m26s_b1_layer_intermediate(const m26s_b1_layer* layer);
 
+/* The prepared pool of a layer, for persisting it or checking it: 256 images of *image_bytes each
+ * (3,342,336 for one rank's share, four times that for a full layer) in expert-id order, device
+ * memory owned by the layer. *layout_tag names the byte order (the counterpart of the reference's
+ * prepared tag, crates/mimo26-expert/kernels/b1/prepared.cuh:16-31): M26S_B1_LAYOUT_G950_V1 is
+ * the operand order of gfx950's v_mfma_scale_f32_16x16x128_f8f6f4 this library writes; a persisted
+ * pool carrying any other tag must be prepared again from the canonical images. Returns 0, or 1
+ * for a null argument. */
+#define M26S_B1_LAYOUT_G950_V1 0x47393501u /* "G95" 0x01 */
+int m26s_b1_layer_view(const m26s_b1_layer* layer, const uint8_t** prepared_dev, uint64_t* image_bytes,
+                       uint32_t* layout_tag);
+
 /* A scratch that launches on the caller's HIP stream (hipStream_t passed as void*; NULL is the
  * default stream) instead of creating its own, so the caller can bracket calls with its own
  * events. The stream is not owned. */

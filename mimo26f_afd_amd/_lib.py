@@ -29,6 +29,7 @@ SIGNATURES = {
     "m26s_b1_ffn": (C.c_int, [_vp, _vp, _vp, _sz, _vp, _sz, _vp, _vp, C.c_uint32, _vp, _vp, _cp, _sz]),
     "m26s_b1_layer_new_full": (C.c_int, [C.POINTER(_vp), C.c_uint64, C.POINTER(_vp), _cp, _sz]),
     "m26s_b1_layer_intermediate": (C.c_uint32, [_vp]),
+    "m26s_b1_layer_view": (C.c_int, [_vp, C.POINTER(_vp), C.POINTER(C.c_uint64), C.POINTER(C.c_uint32)]),
     "m26s_b1_scratch_new_on": (C.c_int, [_vp, C.POINTER(_vp), _cp, _sz]),
     "m26s_b1_ffn_dev": (C.c_int, [_vp, _vp, _vp, _sz, _vp, _sz, _vp, _vp, C.c_uint32, _vp, _vp, _vp, _cp, _sz]),
     "m26s_b1_ffn_enqueue": (C.c_int, [_vp, _vp, _vp, _sz, _vp, _sz, _vp, _vp, C.c_uint32, _vp, _vp, _cp, _sz]),

@@ -74,6 +74,13 @@ class Layer:
     def intermediate(self) -> int:
         return int(load().m26s_b1_layer_intermediate(self._h))
 
+    def prepared_view(self) -> tuple[int, int, int]:
+        """(device pointer of the prepared pool, bytes per expert image, layout tag)."""
+        ptr, nbytes, tag = C.c_void_p(), C.c_uint64(), C.c_uint32()
+        if load().m26s_b1_layer_view(self._h, C.byref(ptr), C.byref(nbytes), C.byref(tag)) != 0:
+            raise B1Error(1, "b1 layer view: bad handle")
+        return int(ptr.value), int(nbytes.value), int(tag.value)
+
     def close(self) -> None:
         if getattr(self, "_h", None) and self._h.value and load is not None:  # load is gone at interpreter exit
             load().m26s_b1_layer_free(self._h)

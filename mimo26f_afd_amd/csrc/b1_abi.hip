@@ -322,6 +322,14 @@ int m26s_b1_layer_new_full(const uint8_t* const rank_images_dev[4], uint64_t byt
 int m26s_b1_layer_all_normal(const m26s_b1_layer* L) { return L && L->all_normal ? 1 : 0; }
 uint32_t m26s_b1_layer_intermediate(const m26s_b1_layer* L) { return L ? L->lay.inter : 0; }
 
+int m26s_b1_layer_view(const m26s_b1_layer* L, const uint8_t** prepared_dev, uint64_t* image_bytes, uint32_t* layout_tag) {
+    if (!L || !prepared_dev || !image_bytes || !layout_tag) return 1;
+    *prepared_dev = L->prepared;
+    *image_bytes = L->lay.bytes();
+    *layout_tag = M26S_B1_LAYOUT_G950_V1;
+    return 0;
+}
+
 void m26s_b1_layer_free(m26s_b1_layer* L) {
     if (!L) return;
     if (L->prepared) (void)hipFree(L->prepared);

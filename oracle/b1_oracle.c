@@ -35,6 +35,12 @@
  *   orc_rank_sum_bf16   - sequential binary32 additions in numpy, data where another order
  *                         differs, and the 1 + 2^-24 + 2^-24 - 1 case a fused sum gets wrong.
  *   orc_bf16_rne_nan    - midpoint, signed-zero, infinity, NaN and subnormal vectors.
+ *   prepared_g950       - (numpy, in b1_oracle.py) the prepared byte order of the gfx950 library as
+ *                         a forward map; pinned by hand-worked coordinates of every region, by
+ *                         being a bijection that keeps the byte multiset, and by the measured
+ *                         operand order of the MFMA itself: the closed-form projections only
+ *                         come out exact on the GPU if every byte sits where the instruction
+ *                         reads it.
  */
 #include "b1_oracle.h"
 #include <float.h>

@@ -178,6 +178,61 @@ def plan(capacity, ids, weights, resident=None, out: Plan | None = None) -> Plan
     return _plan_call(LIB.orc_plan, capacity, ids, weights, resident, out or Plan(capacity))
 
 
+def prepared_g950(images) -> np.ndarray:
+    """One expert's prepared image in the gfx950 operand order, from its one or four canonical
+    quarter-slice images (crates/mimo26-expert/src/slice.rs:45-53), written as a forward map: every
+    canonical byte (projection, row, byte of the row) computes where it goes. The library walks
+    destination cells instead; the reference tests its own permutation the same two-sided way
+    (crates/mimo26-expert/tests/b1/host.cpp:30-67). Raises if the map is not a bijection.
+
+    Destination, I = 512 * len(images) intermediate columns, lane = 16 * (k-block % 4) + row % 16:
+      gate/up payload  [I/32][32 k-steps][4 tiles][64 lanes][16 B], tile = (row % 32) // 16 + (2 for up)
+      gate/up scales   [I/32][8][4 tiles][64 lanes][4 B], byte = k-step % 4 of quad k-step // 4
+      down payload     [64][I/128 k-steps][4 tiles][64 lanes][16 B], tile = (row % 64) // 16
+      down scales      [64][I/512][4 tiles][64 lanes][4 B]
+    with k-block = k // 32 and k-step = k-block // 4; the down projection's K runs over the ranks."""
+    ranks = len(images)
+    inter = 512 * ranks
+    w13, s13 = 0, inter * 4096
+    w2 = s13 + inter * 256
+    s2 = w2 + inter * 2048
+    total = s2 + inter * 128
+    out = np.zeros(total, np.uint8)
+    hits = np.zeros(total, np.uint8)
+
+    def put(dest, values):
+        np.add.at(hits, dest.reshape(-1), 1)
+        out[dest.reshape(-1)] = values.reshape(-1)
+
+    for r, img in enumerate(images):
+        img = np.ascontiguousarray(img, np.uint8)
+        assert img.size == 3342336
+        for up, (pay, sc) in enumerate(((0, 1048576), (1114112, 2162688))):
+            n = (r * 512 + np.arange(512))[:, None]                      # intermediate column
+            b = np.arange(2048)[None, :]                                # byte of the row, 16 per k-block
+            kb, within = b // 16, b % 16
+            lane = 16 * (kb % 4) + n % 16
+            tile = (n % 32) // 16 + 2 * up
+            put(w13 + ((((n // 32) * 32 + kb // 4) * 4 + tile) * 64 + lane) * 16 + within, img[pay:pay + 512 * 2048].reshape(512, 2048))
+            kb = np.arange(128)[None, :]
+            lane = 16 * (kb % 4) + n % 16
+            step = kb // 4
+            put(s13 + ((((n // 32) * 8 + step // 4) * 4 + tile) * 64 + lane) * 4 + step % 4, img[sc:sc + 512 * 128].reshape(512, 128))
+        n = np.arange(4096)[:, None]                                    # output column
+        b = np.arange(256)[None, :]
+        kb, within = r * 16 + b // 16, b % 16
+        lane = 16 * (kb % 4) + n % 16
+        tile = (n % 64) // 16
+        put(w2 + ((((n // 64) * (inter // 128) + kb // 4) * 4 + tile) * 64 + lane) * 16 + within, img[2228224:2228224 + 4096 * 256].reshape(4096, 256))
+        kb = r * 16 + np.arange(16)[None, :]
+        lane = 16 * (kb % 4) + n % 16
+        step = kb // 4
+        put(s2 + ((((n // 64) * (inter // 512) + step // 4) * 4 + tile) * 64 + lane) * 4 + step % 4, img[3276800:3276800 + 4096 * 16].reshape(4096, 16))
+    if not np.all(hits == 1):
+        raise AssertionError("prepared layout: the forward map is not a bijection")
+    return out
+
+
 def silu_up(g, u) -> np.ndarray:
     g = np.asarray(g, np.float32)
     u = np.asarray(u, np.float32)

@@ -6,7 +6,8 @@ import numpy as np
 import pytest
 
 import b1_oracle as O
-from mimo26f_afd_amd import b1
+from helpers import DeviceLayer
+from mimo26f_afd_amd import b1, synth
 
 pytestmark = pytest.mark.gpu
 FIX = np.load(os.path.join(os.path.dirname(__file__), "golden", "b1_host_units.npz"))
@@ -164,3 +165,27 @@ def test_combine_faults(what):
     if what == "product_overflow": y[:] = 0; w[:] = 1; w[0, 0] = 2.0; y[0, 0, 5] = 3.4028235e38
     if what == "sum_overflow": y[:] = 0; w[:] = 1; y[0, :2, 5] = 3.4028235e38
     assert O.reduce(y, w)[0] == 8 and reduce_gpu(y, w)[0] != 0
+
+
+@pytest.mark.parametrize("ranks", [1, 4])
+def test_prepared_pool_is_the_forward_map_of_the_canonical_images(ranks):
+    """The one-time weight preparation, two-sided like the reference's own test of its permutation
+    (crates/mimo26-expert/tests/b1/host.cpp:30-67): the library walks destination cells, the checker
+    maps every canonical byte forward; the prepared images must be identical, for one rank's share and
+    for four ranks fused, on arbitrary bytes (scale bytes included: the permutation moves bytes, it
+    does not read them)."""
+    rng = np.random.default_rng(40 + ranks)
+    pools = [np.full(synth.EXPERTS * synth.IMAGE_BYTES, 0x22, np.uint8) for _ in range(ranks)]
+    experts = (0, 131, 255)
+    for pool in pools:
+        for e in experts:
+            pool[e * synth.IMAGE_BYTES:(e + 1) * synth.IMAGE_BYTES] = rng.integers(0, 256, synth.IMAGE_BYTES, dtype=np.uint8)
+    layer = DeviceLayer(pools).layer
+    assert layer.intermediate == 512 * ranks and not layer.all_scales_normal()
+    ptr, image_bytes, tag = layer.prepared_view()
+    assert image_bytes == ranks * synth.IMAGE_BYTES and tag == 0x47393501
+    for e in experts + (7,):
+        got = np.empty(image_bytes, np.uint8)
+        assert b1.load().m26s_b1_copy_to_host(got.ctypes.data, ptr + e * image_bytes, image_bytes) == 0
+        want = O.prepared_g950([p[e * synth.IMAGE_BYTES:(e + 1) * synth.IMAGE_BYTES] for p in pools])
+        assert np.array_equal(got, want), e
