@@ -9,8 +9,11 @@ from . import build
 _u8p, _f32p, _i32p, _u32p, _u16p = (C.POINTER(t) for t in (C.c_uint8, C.c_float, C.c_int32, C.c_uint32, C.c_uint16))
 _vp, _sz, _cp = C.c_void_p, C.c_size_t, C.c_char_p
 
-# name -> (restype, argtypes); every symbol include/m26s_b1.h, include/m26c_glue.h and include/m26_probe.h declare
+# name -> (restype, argtypes); every symbol include/m26s_b1.h, include/m26c_glue.h, include/m26_probe.h and include/m26w_frame.h declare
 SIGNATURES = {
+    "m26w_crc32c_update": (C.c_uint32, [C.c_uint32, _vp, _sz]),
+    "m26w_request_routes_dev": (C.c_int, [_vp, _vp, C.c_uint32, C.c_uint32, _vp, _vp, _vp, _vp]),
+    "m26w_stage_rows_dev": (C.c_int, [_vp, _vp, _sz, _vp]),
     "m26p_read_bandwidth": (C.c_int, [C.c_uint64, C.c_int, _vp, C.POINTER(C.c_double), _cp, _sz]),
     "m26p_mfma_rate": (C.c_int, [C.c_int, C.c_int, _vp, C.POINTER(C.c_double), _cp, _sz]),
     "m26c_router_topk": (C.c_int, [_vp, _vp, C.c_int, C.c_int, C.c_int, _vp, _vp, _vp]),

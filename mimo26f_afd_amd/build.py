@@ -7,9 +7,9 @@ import subprocess
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB = os.path.join(HERE, "lib", "libm26s_b1.so")
-SOURCES = ["csrc/b1_abi.hip", "csrc/glue_abi.hip", "csrc/probe_abi.hip"]
+SOURCES = ["csrc/b1_abi.hip", "csrc/glue_abi.hip", "csrc/probe_abi.hip", "csrc/frame_abi.hip"]
 DEPENDS = ["csrc/b1_kernels.h", "csrc/b1_tile.h", "csrc/b1_layout.h", "csrc/glue_kernels.h", "../include/m26s_b1.h",
-           "../include/m26c_glue.h", "../include/m26_probe.h"]
+           "../include/m26c_glue.h", "../include/m26_probe.h", "../include/m26w_frame.h"]
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared", "-ffp-contract=off",
          # packed FP32 instructions stay off on this target
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wall", "-Wextra"]
