@@ -419,13 +419,20 @@ __device__ __forceinline__ void fc2_tile_body(const Fc2Args& a, const Chunk ch, 
 
 // Work item of a tile workgroup. Workgroups are handed to the eight XCDs in turn, each with an L2 of
 // its own: the `columns` workgroups of one chunk all take ids of one residue mod 8, so a chunk's
-// activation rows enter one L2 only. The grid is columns * (chunk capacity rounded up to 8).
+// activation rows enter one L2 only, and so do those of the chunk after it: chunks are in expert
+// order, two neighbours mostly share their expert, and their workgroups of one column, dispatched
+// back to back, stream the same weights through that L2 (measured: 2.7 % off FC1 at 8192 tokens; runs
+// of four gained less). The grid is columns * (chunk capacity rounded up to 8 runs).
 struct TileItem { uint32_t chunk, column; };
+constexpr uint32_t kTileRun = 2;  // neighbouring chunks per XCD
 __device__ __forceinline__ TileItem tile_item(uint32_t columns) {
     const uint32_t id = blockIdx.x, xcd = id & 7, slot = id >> 3;
-    return TileItem{(slot / columns) * 8 + xcd, slot % columns};
+    const uint32_t per = columns * kTileRun, run = slot / per, within = slot % per;
+    return TileItem{(run * 8 + xcd) * kTileRun + within % kTileRun, within / kTileRun};
 }
-__host__ inline uint32_t tile_grid(uint32_t columns, uint32_t chunk_cap) { return columns * ((chunk_cap + 7) / 8 * 8); }
+__host__ inline uint32_t tile_grid(uint32_t columns, uint32_t chunk_cap) {
+    return columns * ((chunk_cap + 8 * kTileRun - 1) / (8 * kTileRun) * (8 * kTileRun));
+}
 
 // 256 threads, one workgroup per (chunk, 128 intermediate columns). Chunks of one or two groups run
 // the register-only bodies (each wave is independent there); larger chunks share activations
