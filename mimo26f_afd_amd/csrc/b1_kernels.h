@@ -397,12 +397,14 @@ plan_scan_kernel(uint32_t routes, uint32_t* __restrict__ work, PlanView p, uint3
     const uint32_t e = tid & 255, quarter = tid >> 8, per = (waves + 3) / 4;
     const uint32_t k0 = quarter * per, k1 = k0 + per < waves ? k0 + per : waves;
     uint32_t sum = 0;
-    for (uint32_t k = k0; k < k1; ++k) sum += counts[uint64_t(k) * 256 + e];
+#pragma unroll 16
+    for (uint32_t k = k0; k < k1; ++k) sum += counts[uint64_t(k) * 256 + e];  // unrolled: the loads are independent, the walk is latency
     part[quarter][e] = sum;
     __syncthreads();
     uint32_t run = 0;
     for (uint32_t qd = 0; qd < quarter; ++qd) run += part[qd][e];
     if (quarter == 3) cnt[e] = run + sum;
+#pragma unroll 16
     for (uint32_t k = k0; k < k1; ++k) {
         const uint32_t c = counts[uint64_t(k) * 256 + e];
         counts[uint64_t(k) * 256 + e] = run;
