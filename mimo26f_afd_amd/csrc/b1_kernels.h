@@ -823,8 +823,8 @@ template <int NT>
 __global__ void __launch_bounds__(256) fc1_kernel(Fc1Args a) {
     uint32_t* meta = a.plan.meta;
     const uint32_t c = blockIdx.y;
+    const Chunk ch = a.plan.chunks[c];  // fetched beside the verdict words, not after them (the table covers the whole grid)
     if (meta[kPlanFault] || c >= meta[kChunkCount]) return;
-    const Chunk ch = a.plan.chunks[c];
     const uint32_t lane = threadIdx.x & 63, cb = blockIdx.x * 4 + (threadIdx.x >> 6);
     const int32_t expert = ch.expert;
     if (expert < 0 || expert >= int32_t(kExperts) || ch.groups < 1 || ch.groups > NT) {
@@ -906,8 +906,8 @@ template <int NT>
 __global__ void __launch_bounds__(256) fc2_kernel(Fc2Args a) {
     uint32_t* meta = a.plan.meta;
     const uint32_t c = blockIdx.y;
+    const Chunk ch = a.plan.chunks[c];  // fetched beside the verdict words, not after them
     if (meta[kPlanFault] || meta[kFc1Fault] || meta[kQuantFault] || c >= meta[kChunkCount]) return;
-    const Chunk ch = a.plan.chunks[c];
     const uint32_t lane = threadIdx.x & 63, ob = blockIdx.x * 4 + (threadIdx.x >> 6);
     const int32_t expert = ch.expert;
     if (expert < 0 || expert >= int32_t(kExperts) || ch.groups < 1 || ch.groups > NT) {
