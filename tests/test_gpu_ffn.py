@@ -242,6 +242,36 @@ def test_prefill_chunk_properties_and_sampled_parity(full_layer):
     assert np.array_equal(bf_p, bf[perm])
 
 
+def test_maximum_rows_on_eight_experts():
+    """The largest call (8192 rows) with every token routed to the same eight experts: 8192 rows per
+    expert, 64 full chunks each, the collision the planner's counters and the tile schedule see at most.
+    Plan bit-exact; sampled rows to the bars; rows of identical input and routes come out identical."""
+    seed, rows = synth.BASE_SEED + 21, 8192
+    experts = [5, 40, 77, 101, 130, 188, 200, 255]
+    rng = np.random.default_rng(21)
+    ids = np.stack([rng.permutation(experts) for _ in range(rows)]).astype(np.int32)
+    w, x = synth._softmax_weights(seed, rows), synth._activations(seed, rows)
+    x[4096:] = x[:4096]                                                     # second half repeats the first ...
+    ids[4096:], w[4096:] = ids[:4096], w[:4096]                             # ... routes and weights included
+    payload, scales = synth.q0_quantize(x)
+    wl = synth.Workload("eight experts", 1, seed, 1, rows, ids, w, x, payload, scales)
+    pools = [synth.rank_pool(seed, 0, experts)]
+    layer = DeviceLayer(pools).layer
+    s = b1.Scratch()
+    stats, bf, pf = run_ffn_dev(layer, s, wl)
+    n = rows * 8
+    ref = O.plan(8192, ids, w)
+    assert ref.status == 0 and stats.groups == int(ref.group_count[0]) == 8 * 512
+    assert np.array_equal(s.view("original_routes", np.int32, n), ref.original_routes[:n])
+    assert np.array_equal(s.view("inverse", np.int32, n), ref.inverse[:n])
+    assert np.array_equal(s.view("groups", O.GROUP_DTYPE, stats.groups), ref.groups[:stats.groups])
+    assert np.array_equal(bf[4096:], bf[:4096]) and np.array_equal(pf[4096:].view(np.uint32), pf[:4096].view(np.uint32))
+    sample = np.array([0, 1, 2047, 4095, 4096, 6000, 8190, 8191])
+    rc, ref_partial, ref_bf16, _ = O.layer_ffn(pools, payload[sample], scales[sample], ids[sample], w[sample])
+    assert rc == 0
+    check_outputs(pf[sample], bf[sample], ref_partial, ref_bf16)
+
+
 def test_errors_and_faults(full_layer):
     """Return codes and messages of the reference entry (b1_serve.cu:315-317,365,551-562)."""
     wl, pools, layer = full_layer
