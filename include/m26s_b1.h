@@ -118,6 +118,15 @@ int m26s_b1_reduce_dev(const float* y_dev, const float* weights_dev, uint32_t ro
 
 /* With taps on, the next FFN calls also keep FP32 gate / up / h of every grouped row. */
 void m26s_b1_scratch_set_taps(m26s_b1_scratch* scratch, int on);
+/* No counterpart in the reference. Off by default. When on, prefill-size calls (more than 128 rows) on
+ * a full-intermediate layer run FC2's chunks of five to eight groups through one persistent
+ * eight-wave workgroup per compute unit (operands in one pipeline across work items, the finished
+ * accumulators stored under the next item's MFMAs) and leave the smaller chunks to the tile kernel.
+ * Results are bit for bit those of the default schedule; at 8192 tokens it is measured slower
+ * (0.85 against 0.75 ms: FC2 is bound by the writes of the per-route rows either way, and the small
+ * chunks no longer overlap the large ones), so it is kept as the tested base of the FC1 kernel of the
+ * same shape, not as the serving path. */
+void m26s_b1_scratch_set_stream(m26s_b1_scratch* scratch, int on);
 /* Device address and byte size of an internal buffer after a call. which: 0 inverse, 1 original
  * routes, 2 grouped weights, 3 groups, 4 meta words {group count, plan fault, chunk count, fc1
  * fault, quantizer fault, lowest faulting block, fc2 fault, reduce fault}, 5 intermediate payload

@@ -1,18 +1,22 @@
-"""Check of the tile kernels' generated code around their hand-issued loads.
+"""Check of the tile and stream kernels' generated code around their hand-issued loads.
 
-The k-loop of csrc/b1_tile.h issues its scale loads and LDS reads as `asm` statements and orders them
-with explicit s_waitcnt, because a load the compiler knows of makes it drain the direct-to-LDS
-prefetch. The price: to the compiler such a register holds its value the moment the instruction has
-issued. Two things must therefore hold in the generated code, and this module checks them on the
-assembly hipcc emits (no GPU needed):
+The k-loops of csrc/b1_tile.h and csrc/b1_stream.h issue their scale loads, route lookups and LDS
+reads as `asm` statements and order them with explicit s_waitcnt, because a load the compiler knows
+of makes it drain the direct-to-LDS prefetch. The price: to the compiler such a register holds its
+value the moment the instruction has issued. Two things must therefore hold in the generated code,
+and this module checks them on the assembly hipcc emits (no GPU needed):
 
- 1. a register with a hand-issued load in flight is read by nothing but an MFMA (behind the waits the
-    source places), and
- 2. it is not written by a compiler instruction before an MFMA has read it or a closing
-    `s_waitcnt vmcnt(0)` / `lgkmcnt(0)` has passed: the data in flight would land on top of the new
-    value (an address, say).
+ 1. a register with a hand-issued load in flight is not read, and
+ 2. it is not written: the data in flight would land on top of the new value (an address, say).
 
-Each tile kernel is walked in layout order, twice (loops wrap), which is conservative for the
+"In flight" follows the hardware's counters. Vector-memory operations (loads, stores, direct-to-LDS
+loads, whoever issued them) complete in issue order, and `s_waitcnt vmcnt(N)` returns when at most N
+are outstanding: the checker keeps them in a queue and retires all but the newest N at such a wait.
+LDS reads retire at `lgkmcnt(0)`, the only form the kernels use. An MFMA also retires the registers
+it reads: the sources place every MFMA behind the wait for its operands, and the queue model then
+agrees.
+
+Each kernel is walked in layout order, twice (loops wrap), which is conservative for the
 straight-line tails. `python -m mimo26f_afd_amd.codegen_check` compiles and checks.
 """
 from __future__ import annotations
@@ -37,11 +41,15 @@ def _regs(tok: str) -> set:
     return {int(m.group(1))} if m else set()
 
 
+VM_PREFIX = ("global_load", "global_store", "global_atomic", "buffer_", "scratch_", "flat_")
+KERNELS = r"^(_ZN4m26g\w*(?:tile|stream)_kernel\w*):"
+
+
 def check(asm_text: str) -> tuple[dict, list]:
     """Returns ({kernel: hand-issued loads seen}, [problem lines])."""
     funcs, name = {}, None
     for line in asm_text.split("\n"):
-        m = re.match(r"^(_ZN4m26g\w*tile_kernel\w*):", line)
+        m = re.match(KERNELS, line)
         if m:
             name = m.group(1)
             funcs[name] = []
@@ -52,7 +60,7 @@ def check(asm_text: str) -> tuple[dict, list]:
             funcs[name].append(line)
     seen, problems = {}, []
     for fn, body in funcs.items():
-        flying_vm, flying_lds, inasm, loads = set(), set(), False, 0
+        vm_queue, flying_lds, inasm, loads = [], set(), False, 0
         for line in body + body:
             if "ASMSTART" in line:
                 inasm = True
@@ -65,29 +73,43 @@ def check(asm_text: str) -> tuple[dict, list]:
                 continue
             op = tok[0]
             if op == "s_waitcnt":
-                if "vmcnt(0)" in line:
-                    flying_vm.clear()
+                m = re.search(r"vmcnt\((\d+)\)", line)
+                if m:
+                    del vm_queue[:max(0, len(vm_queue) - int(m.group(1)))]
                 if "lgkmcnt(0)" in line:
                     flying_lds.clear()
                 continue
+            flying = flying_lds.union(*vm_queue) if vm_queue else set(flying_lds)
             if inasm:
                 if op.startswith("ds_read"):
                     flying_lds |= _regs(tok[1])
                     loads += 1
-                elif op == "global_load_dword":
-                    flying_vm |= _regs(tok[1])
+                elif op.startswith("global_load_dword") and not op.startswith("global_load_lds"):
+                    vm_queue.append(_regs(tok[1]))
                     loads += 1
+                elif op.startswith(VM_PREFIX):
+                    vm_queue.append(set())
                 elif op.startswith("v_mfma"):
+                    used = set()
                     for t in tok[2:]:
-                        flying_vm -= _regs(t)
-                        flying_lds -= _regs(t)
+                        used |= _regs(t)
+                    flying_lds -= used
+                    for entry in vm_queue:
+                        entry -= used
+                elif op.startswith(("ds_write", "v_accvgpr")):
+                    srcs = set()
+                    for t in tok[1:]:
+                        srcs |= _regs(t)
+                    if srcs & flying:
+                        problems.append(f"{fn}: hand-written instruction reads a register with a load in flight: {line.strip()}")
                 continue
+            if op.startswith(VM_PREFIX):
+                vm_queue.append(set())  # the compiler's own: it waits for them itself, but they hold a place in the order
             nodest = op.startswith(NO_DEST)
             dest = set() if nodest or len(tok) < 2 else _regs(tok[1])
             srcs = set()
             for t in tok[(1 if nodest else 2):]:
                 srcs |= _regs(t)
-            flying = flying_vm | flying_lds
             if srcs & flying:
                 problems.append(f"{fn}: reads a register with a hand-issued load in flight: {line.strip()}")
             if dest & flying:
@@ -111,8 +133,8 @@ def compile_to_asm() -> str:
 def run() -> dict:
     """Compile, check, raise on any problem; returns the per-kernel count of hand-issued loads."""
     seen, problems = check(compile_to_asm())
-    if len(seen) < 2 or min(seen.values()) < 100:
-        raise RuntimeError(f"codegen check: tile kernels not found in the assembly ({seen})")
+    if len(seen) < 3 or min(seen.values()) < 100:
+        raise RuntimeError(f"codegen check: tile and stream kernels not found in the assembly ({seen})")
     if problems:
         raise RuntimeError("codegen check failed:\n" + "\n".join(problems[:12]))
     return seen

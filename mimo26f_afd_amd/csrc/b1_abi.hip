@@ -11,7 +11,7 @@
 #include <vector>
 
 #include "../../include/m26s_b1.h"
-#include "b1_tile.h"
+#include "b1_stream.h"
 
 using namespace m26g;
 
@@ -57,6 +57,7 @@ uint32_t tiles_for(uint32_t rows) { return rows <= 32 ? 1u : rows <= 128 ? 2u : 
 
 // Kernels whose dynamic LDS passes 64 KB need the limit raised once per process.
 bool lds_ready = false;
+uint32_t compute_units = 0;  // of the device the first scratch was made on
 hipError_t plan_lds_attr() {
     if (lds_ready) return hipSuccess;
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(plan_kernel),
@@ -67,6 +68,13 @@ hipError_t plan_lds_attr() {
     if (e == hipSuccess)
         e = hipFuncSetAttribute(reinterpret_cast<const void*>(fc2_tile_kernel),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, int(kTileLdsBytes));
+    if (e == hipSuccess)
+        e = hipFuncSetAttribute(reinterpret_cast<const void*>(fc2_stream_kernel),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, int(kStreamLdsBytes));
+    int device = 0, cus = 0;
+    if (e == hipSuccess) e = hipGetDevice(&device);
+    if (e == hipSuccess) e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device);
+    compute_units = uint32_t(cus);
     lds_ready = e == hipSuccess;
     return e;
 }
@@ -84,9 +92,10 @@ struct m26s_b1_scratch {
     hipStream_t st = nullptr;
     bool own_stream = false;
     hipEvent_t e0 = nullptr, ep = nullptr, ea = nullptr, ec = nullptr, e1 = nullptr;
-    Dev x, xs, iw, inv, orig, gw, groups, chunks, meta, dq, dqs, y, bf16, pad, tap_gate, tap_up, tap_h, xg, rowbad, dg, planw, xrows, yrows;
+    Dev x, xs, iw, inv, orig, gw, groups, chunks, meta, dq, dqs, y, bf16, pad, tap_gate, tap_up, tap_h, xg, rowbad, dg, planw, xrows, yrows, big;
     std::vector<uint8_t> hiw;
     bool taps = false;
+    bool stream_fc2 = false;  // FC2's large chunks through the persistent kernel of b1_stream.h
     uint32_t last_rows = 0, last_inter = 0;
 };
 
@@ -163,7 +172,7 @@ void launch_ffn(const m26s_b1_layer* L, m26s_b1_scratch* S, const PlanView& pv, 
     fc1_kernel<NT><<<dim3(L->lay.inter / 128, chunk_cap), 256, 0, S->st>>>(f1);
     (void)hipEventRecord(S->ea, S->st);
     Fc2Args f2{L->prepared, L->lay, pv, S->dq.as<uint8_t>(), S->dqs.as<uint8_t>(), zero, zero + 8192,
-               S->y.as<float>(), uint32_t(routes), nullptr, nullptr, nullptr};
+               S->y.as<float>(), uint32_t(routes), nullptr, nullptr, nullptr, 0};
     fc2_kernel<NT><<<dim3(16, chunk_cap), 256, 0, S->st>>>(f2);
     (void)hipEventRecord(S->ec, S->st);
 }
@@ -173,8 +182,11 @@ void launch_tiles(const m26s_b1_layer* L, m26s_b1_scratch* S, const PlanView& pv
                   const uint8_t* xs, size_t xsp, uint32_t chunk_cap, uint64_t routes) {
     const uint8_t* zero = S->pad.as<uint8_t>();
     const uint32_t inter = L->lay.inter;
+    // Full-intermediate layers hand FC2's large chunks to the persistent stream kernel (b1_stream.h).
+    const bool stream = S->stream_fc2 && inter == kStreamSteps * 128 && compute_units >= 8;
     gather_scales_kernel<<<chunk_cap, 256, 0, S->st>>>(pv, xs, xsp, S->xg.as<uint32_t>(), S->rowbad.as<uint32_t>(),
-                                                     S->xrows.as<int32_t>(), S->yrows.as<int32_t>());
+                                                     S->xrows.as<int32_t>(), S->yrows.as<int32_t>(),
+                                                     stream ? S->big.as<int32_t>() : nullptr);
     Fc1Args f1{L->prepared, L->lay, pv, x, xp, xs, xsp, zero, zero + 8192, S->dq.as<uint8_t>(), S->dqs.as<uint8_t>(),
                S->taps ? S->tap_gate.as<float>() : nullptr, S->taps ? S->tap_up.as<float>() : nullptr,
                S->taps ? S->tap_h.as<float>() : nullptr, S->xg.as<uint8_t>(), S->rowbad.as<uint32_t>(), S->xrows.as<int32_t>(),
@@ -182,7 +194,11 @@ void launch_tiles(const m26s_b1_layer* L, m26s_b1_scratch* S, const PlanView& pv
     fc1_tile_kernel<<<tile_grid(inter / 128, chunk_cap), kTileThreads, kTileLdsBytes, S->st>>>(f1);
     (void)hipEventRecord(S->ea, S->st);
     Fc2Args f2{L->prepared, L->lay, pv, S->dq.as<uint8_t>(), S->dqs.as<uint8_t>(), zero, zero + 8192,
-               S->y.as<float>(), uint32_t(routes), S->dg.as<uint8_t>(), S->yrows.as<int32_t>(), S->rowbad.as<uint32_t>()};
+               S->y.as<float>(), uint32_t(routes), S->dg.as<uint8_t>(), S->yrows.as<int32_t>(), S->rowbad.as<uint32_t>(), 0};
+    if (stream) {
+        fc2_stream_kernel<<<compute_units / 8 * 8, kStreamThreads, kStreamLdsBytes, S->st>>>(StreamArgs{f2, S->big.as<BigChunk>()});
+        f2.skip_from = kStreamFromGroups;
+    }
     fc2_tile_kernel<<<tile_grid(kHidden / 256, chunk_cap), kTileThreads, kTileLdsBytes, S->st>>>(f2);
     (void)hipEventRecord(S->ec, S->st);
 }
@@ -200,15 +216,18 @@ int enqueue(const m26s_b1_layer* L, m26s_b1_scratch* S, const uint8_t* x, size_t
     M26S_CK(S->gw.ensure(route_cap * 4), "b1 gw alloc");
     M26S_CK(S->groups.ensure(route_cap * sizeof(Group)), "b1 groups alloc");
     M26S_CK(S->chunks.ensure(route_cap * sizeof(Chunk)), "b1 chunks alloc");
-    M26S_CK(S->dq.ensure(gcap * 16 * inter), "b1 dq alloc");
+    // Eight groups of slack behind the intermediate and one spare row behind y: the stream kernel reads
+    // all eight tiles of a chunk whatever its group count, and parks the rows that hold no token.
+    M26S_CK(S->dq.ensure((gcap + 8) * 16 * inter), "b1 dq alloc");
     M26S_CK(S->dqs.ensure(gcap * 16 * inter / 32), "b1 dqs alloc");
-    M26S_CK(S->y.ensure(routes * kHidden * 4), "b1 y alloc");
+    M26S_CK(S->y.ensure((routes + 1) * kHidden * 4), "b1 y alloc");
     if (nt > 2) {
         M26S_CK(S->xg.ensure(ccap * gathered_scale_bytes(kHidden)), "b1 gathered input scales alloc");
         M26S_CK(S->dg.ensure(ccap * gathered_scale_bytes(inter)), "b1 gathered intermediate scales alloc");
         M26S_CK(S->rowbad.ensure(ccap * 16 * 4), "b1 row verdict alloc");
         M26S_CK(S->xrows.ensure(ccap * 128 * 4), "b1 chunk row table alloc");
         M26S_CK(S->yrows.ensure(ccap * 128 * 4), "b1 chunk route table alloc");
+        M26S_CK(S->big.ensure((ccap + 1) * sizeof(BigChunk)), "b1 large chunk list alloc");
     }
     if (S->taps) {
         M26S_CK(S->tap_gate.ensure(gcap * 16 * inter * 4), "b1 gate tap alloc");
@@ -482,6 +501,7 @@ int m26s_b1_reduce_dev(const float* y_dev, const float* weights_dev, uint32_t ro
     return 0;
 }
 
+void m26s_b1_scratch_set_stream(m26s_b1_scratch* S, int on) { if (S) S->stream_fc2 = on != 0; }
 void m26s_b1_scratch_set_taps(m26s_b1_scratch* S, int on) { if (S) S->taps = on != 0; }
 
 int m26s_b1_scratch_view(const m26s_b1_scratch* S, int which, void** dev_ptr, size_t* bytes) {

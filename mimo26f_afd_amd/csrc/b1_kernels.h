@@ -850,6 +850,7 @@ struct Fc2Args {
     const uint8_t* dg;  // tile schedule only: the intermediate's scales in MFMA lane order (see Fc1Args)
     const int32_t* yrows;  // tile schedule only, [chunk][8 tiles][16]: the route (row of y) of each row, -1 for none
     const uint32_t* rowbad;  // tile schedule only: as in Fc1Args (bit 8+t: tile t holds a token in that row)
+    int32_t skip_from;       // tile schedule only: chunks of at least this many groups belong to the stream kernel (0: none)
 };
 
 // FC2 epilogue of one wave: unweighted FP32 rows back to y[original route].

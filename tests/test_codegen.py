@@ -34,4 +34,4 @@ def test_checker_flags_reads_and_writes_under_a_load_in_flight():
 
 def test_built_tile_kernels_pass():
     seen = codegen_check.run()
-    assert len(seen) == 2 and all(n >= 100 for n in seen.values())
+    assert len(seen) == 3 and all(n >= 100 for n in seen.values())

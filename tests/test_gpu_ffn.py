@@ -242,6 +242,27 @@ def test_prefill_chunk_properties_and_sampled_parity(full_layer):
     assert np.array_equal(bf_p, bf[perm])
 
 
+def test_stream_schedule_gives_the_default_schedule_bits(full_layer):
+    """The persistent FC2 kernel for chunks of five to eight groups (off by default) reproduces the
+    default schedule bit for bit: configs[3] at 8192 tokens, then a ragged 1000 tokens on the same
+    scratch (smaller second call: few large chunks, most of the work left to the tile kernel)."""
+    _, _, layer = full_layer
+    wl = synth.make(3)
+    pick = np.arange(1000) * 7 % wl.rows
+    small = synth.Workload("ragged", 3, wl.seed, 4, len(pick), wl.ids[pick], wl.weights[pick], wl.x[pick],
+                           wl.payload[pick], wl.scales[pick])
+    s = b1.Scratch()
+    base = [run_ffn_dev(layer, s, w) for w in (wl, small)]
+    s.set_stream(True)
+    for w, (stats0, bf0, pf0) in zip((wl, small), base):
+        stats, bf, pf = run_ffn_dev(layer, s, w)
+        assert stats.groups == stats0.groups
+        assert np.array_equal(bf, bf0) and np.array_equal(pf.view(np.uint32), pf0.view(np.uint32))
+    s.set_stream(False)
+    _, bf, _ = run_ffn_dev(layer, s, small, want_partial=False)
+    assert np.array_equal(bf, base[1][1])
+
+
 def test_maximum_rows_on_eight_experts():
     """The largest call (8192 rows) with every token routed to the same eight experts: 8192 rows per
     expert, 64 full chunks each, the collision the planner's counters and the tile schedule see at most.
