@@ -26,8 +26,8 @@ MFMA_FP8_PEAK_TFLOPS = 5000.0   # dense FP8 (an FP8 x FP4 block-scaled MFMA issu
 # HBM bytes per launch of the dominant kernels on these workloads, from two rocprofv3 --pmc runs of this
 # file (FETCH_SIZE, WRITE_SIZE), each scaled by what the same counter reads for --copy-probe's 1 GiB copy:
 # one FETCH_SIZE count = 2.0 KiB, one WRITE_SIZE count = 1.0 KiB.
-FC1_DECODE_TRAFFIC_BYTES = int((2.0 * 857876 + 1.0 * 2570) * 1024)
-FC1_PREFILL_TRAFFIC_BYTES = int((2.0 * 2764413 + 1.0 * 142260) * 1024)
+FC1_DECODE_TRAFFIC_BYTES = int((2.0 * 857916 + 1.0 * 2570) * 1024)
+FC1_PREFILL_TRAFFIC_BYTES = int((2.0 * 2332868 + 1.0 * 140311) * 1024)
 
 
 def log(*a):
