@@ -34,7 +34,6 @@ constexpr int kStreamThreads = 512, kStreamWaves = 8, kStreamStages = 3, kStream
 constexpr uint32_t kStreamWeightRing = 4 * kStreamStages * 4096, kStreamActRing = kStreamStages * 16384;
 constexpr uint32_t kStreamStrip = 16 * 272;
 constexpr uint32_t kStreamLdsBytes = kStreamWeightRing + kStreamActRing + kStreamWaves * kStreamStrip;
-constexpr int32_t kStreamFromGroups = 5;  // chunks of at least this many groups take this kernel
 
 // A large chunk as the stream kernel wants it: everything one scalar load away from the item index.
 struct BigChunk { int32_t chunk, expert, first_group, groups; };

@@ -36,6 +36,7 @@ namespace m26g {
 constexpr int kTileThreads = 256, kTileWaves = 4, kWeightStages = 2, kActStages = 3;
 constexpr uint32_t kTileLdsBytes = kTileWaves * kWeightStages * 4096 + kActStages * 8 * 2048;
 static_assert(kTileLdsBytes == 80 * 1024, "two workgroups share the 160 KB of a compute unit");
+constexpr int32_t kStreamFromGroups = 5;  // chunks of at least this many groups can go to the stream kernel (b1_stream.h)
 // Bytes of one chunk's gathered activation scales for a K-deep product: [K/512][8][64] dwords.
 __host__ __device__ constexpr uint32_t gathered_scale_bytes(uint32_t k) { return (k / 512) * 2048; }
 
@@ -105,7 +106,7 @@ __global__ void __launch_bounds__(256) gather_scales_kernel(PlanView plan, const
         __syncthreads();
         uint32_t mine_before = 0, mine_total = 0;
         for (uint32_t i = tid; i < plan.meta[kChunkCount]; i += 256) {
-            const uint32_t large = plan.chunks[i].groups >= 5 ? 1u : 0u;
+            const uint32_t large = plan.chunks[i].groups >= kStreamFromGroups ? 1u : 0u;
             mine_total += large;
             mine_before += i < c ? large : 0u;
         }
@@ -113,7 +114,7 @@ __global__ void __launch_bounds__(256) gather_scales_kernel(PlanView plan, const
         if (mine_before) atomicAdd(&before, mine_before);
         __syncthreads();
         if (tid == 0) {
-            if (ch.groups >= 5) *reinterpret_cast<int4*>(big + 4 + 4 * before) = int4{int32_t(c), ch.expert, ch.first_group, ch.groups};
+            if (ch.groups >= kStreamFromGroups) *reinterpret_cast<int4*>(big + 4 + 4 * before) = int4{int32_t(c), ch.expert, ch.first_group, ch.groups};
             if (c == 0) big[0] = int32_t(total);
         }
     }
