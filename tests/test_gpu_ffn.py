@@ -263,6 +263,34 @@ def test_stream_schedule_gives_the_default_schedule_bits(full_layer):
     assert np.array_equal(bf, base[1][1])
 
 
+def test_two_scratches_in_flight_on_one_layer(full_layer):
+    """One scratch is one call in flight; two scratches (two streams) may run at once on the same layer.
+    Calls of three sizes (decode schedule, tile schedule) are enqueued alternately without a wait in
+    between; every output equals the one the same call gives alone, bit for bit."""
+    wl, _, layer = full_layer
+    big = synth.make(3)
+    pick = np.arange(700) * 11 % big.rows
+    tile = synth.Workload("tile", 3, big.seed, 4, len(pick), big.ids[pick], big.weights[pick], big.x[pick],
+                          big.payload[pick], big.scales[pick])
+    few = synth.Workload("few", 2, wl.seed, 4, 5, wl.ids[:5], wl.weights[:5], wl.x[:5], wl.payload[:5], wl.scales[:5])
+    calls = [wl, tile, few, tile, wl, few]
+    alone = b1.Scratch()
+    want = [run_ffn_dev(layer, alone, w, want_partial=False)[1] for w in calls]
+    scratches = [b1.Scratch(), b1.Scratch()]
+    held = []
+    for n, w in enumerate(calls):
+        bufs = [b1.DeviceBuffer.from_host(a) for a in (w.payload, w.scales, w.ids, w.weights)]
+        out = b1.DeviceBuffer(w.rows * 4096 * 2)
+        if n >= 2:
+            scratches[n % 2].sync()                                        # the scratch's previous call, not the other's
+        b1.ffn_enqueue(layer, scratches[n % 2], bufs[0].ptr, 4096, bufs[1].ptr, 128, bufs[2].ptr, bufs[3].ptr, w.rows, out.ptr)
+        held.append((bufs, out))
+    for s in scratches:
+        s.sync()
+    for (bufs, out), w, ref in zip(held, calls, want):
+        assert np.array_equal(out.to_host(np.uint16).reshape(w.rows, 4096), ref)
+
+
 def test_maximum_rows_on_eight_experts():
     """The largest call (8192 rows) with every token routed to the same eight experts: 8192 rows per
     expert, 64 full chunks each, the collision the planner's counters and the tile schedule see at most.
