@@ -32,6 +32,26 @@ def test_checker_flags_reads_and_writes_under_a_load_in_flight():
     assert p == []
 
 
+def test_checker_retires_vector_memory_operations_in_issue_order():
+    """`vmcnt(N)` leaves the newest N operations in flight, stores and direct-to-LDS loads included."""
+    a = hand("global_load_dword v7, v[2:3], off")
+    b = hand("global_load_dword v8, v[2:3], off offset:4")
+    store = "\tglobal_store_dword v[2:3], v1, off"
+    one = hand("s_waitcnt vmcnt(1)")
+    done = hand("s_waitcnt vmcnt(0)")
+    _, p = codegen_check.check(asm(a, b, one, "\tv_add_u32_e32 v9, v7, v1", done))
+    assert p == []                                                       # the older load has landed
+    _, p = codegen_check.check(asm(a, b, one, "\tv_add_u32_e32 v9, v8, v1", done))
+    assert p and "reads" in p[0]                                         # the younger one has not
+    _, p = codegen_check.check(asm(a, b, store, one, "\tv_add_u32_e32 v9, v8, v1", done))
+    assert p == []                                                       # the store is the one left in flight
+    lds_load = hand("global_load_lds_dwordx4 v[2:3], off")
+    _, p = codegen_check.check(asm(a, lds_load, lds_load, hand("s_waitcnt vmcnt(2)"), "\tv_add_u32_e32 v9, v7, v1", done))
+    assert p == []
+    _, p = codegen_check.check(asm(a, lds_load, lds_load, hand("s_waitcnt vmcnt(3)"), "\tv_add_u32_e32 v9, v7, v1", done))
+    assert p and "reads" in p[0]
+
+
 def test_built_tile_kernels_pass():
     seen = codegen_check.run()
     assert len(seen) == 3 and all(n >= 100 for n in seen.values())
