@@ -224,8 +224,10 @@ int enqueue(const m26s_b1_layer* L, m26s_b1_scratch* S, const uint8_t* x, size_t
     if (nt > 2) {
         M26S_CK(S->xg.ensure(ccap * gathered_scale_bytes(kHidden)), "b1 gathered input scales alloc");
         M26S_CK(S->dg.ensure(ccap * gathered_scale_bytes(inter)), "b1 gathered intermediate scales alloc");
-        M26S_CK(S->rowbad.ensure(ccap * 16 * 4), "b1 row verdict alloc");
-        M26S_CK(S->xrows.ensure(ccap * 128 * 4), "b1 chunk row table alloc");
+        // The tile kernels fetch these beside their chunk record, before they know whether the chunk exists:
+        // the tables cover the whole grid (chunk capacity rounded up to runs on eight XCDs).
+        M26S_CK(S->rowbad.ensure((ccap + 8 * kTileRun) * 16 * 4), "b1 row verdict alloc");
+        M26S_CK(S->xrows.ensure((ccap + 8 * kTileRun) * 128 * 4), "b1 chunk row table alloc");
         M26S_CK(S->yrows.ensure(ccap * 128 * 4), "b1 chunk route table alloc");
         M26S_CK(S->big.ensure((ccap + 1) * sizeof(BigChunk)), "b1 large chunk list alloc");
     }

@@ -329,19 +329,17 @@ __device__ __forceinline__ uint32_t after_loop(uint32_t lane) {
 }
 
 // FC1 for chunk c by one workgroup: 128 intermediate columns x 16*TT rows; the wave owns block cb.
+// `token[m]` is the row table's entry for this lane's row of tile wv*(TT/4)+m, fetched by the caller beside
+// the chunk record so that the rows' addresses are one memory latency behind the workgroup's start, not two.
 template <int TT>
 __device__ __forceinline__ void fc1_tile_body(const Fc1Args& a, const Chunk ch, uint32_t c, uint32_t cb, uint32_t wv,
-                                              uint32_t lane, uint8_t* lds) {
+                                              uint32_t lane, uint8_t* lds, const int32_t (&token)[TT / kTileWaves]) {
     constexpr int kMine = TT / kTileWaves;
-    const uint32_t r = lane & 15, g = lane >> 4;
+    const uint32_t g = lane >> 4;
     const int32_t expert = ch.expert;
     const uint8_t* row[kMine];
 #pragma unroll
-    for (int m = 0; m < kMine; ++m) {
-        const int lt = int(wv) * kMine + m;
-        const int32_t mine = a.xrows[c * 128 + lt * 16 + r];
-        row[m] = (mine >= 0 ? a.x + size_t(mine) * a.x_pitch : a.zero_row) + g * 16;
-    }
+    for (int m = 0; m < kMine; ++m) row[m] = (token[m] >= 0 ? a.x + size_t(token[m]) * a.x_pitch : a.zero_row) + g * 16;
     const uint8_t* img = a.prepared + uint64_t(expert) * a.lay.bytes();
     const uint8_t* wp = img + a.lay.w13() + uint64_t(cb) * (32 * 4096) + lane * 16;
     const uint8_t* sp = img + a.lay.s13() + uint64_t(cb) * (8 * 1024) + lane * 4;
@@ -387,13 +385,14 @@ __device__ __forceinline__ void fc1_tile_body(const Fc1Args& a, const Chunk ch, 
 }
 
 // FC2 for chunk c by one workgroup: 256 output columns x 16*TT rows; the wave owns block ob.
+// `verdict` is rowbad[c][lane % 16] (bit 8+t: tile t holds a token in this row), fetched by the caller beside
+// the chunk record.
 template <int TT>
 __device__ __forceinline__ void fc2_tile_body(const Fc2Args& a, const Chunk ch, uint32_t c, uint32_t ob, uint32_t wv,
-                                              uint32_t lane, uint8_t* lds) {
+                                              uint32_t lane, uint8_t* lds, const uint32_t verdict) {
     constexpr int kMine = TT / kTileWaves;
     const uint32_t r = lane & 15, g = lane >> 4, I = a.lay.inter;
     const int32_t expert = ch.expert;
-    const uint32_t verdict = a.rowbad[c * 16 + r];  // bit 8+t: tile t holds a token in this row
     const uint8_t* row[kMine];
 #pragma unroll
     for (int m = 0; m < kMine; ++m) {
@@ -472,8 +471,12 @@ __global__ void __launch_bounds__(kTileThreads, 2) fc1_tile_kernel(Fc1Args a) {
     const TileItem it = tile_item(a.lay.inter / 128);
     const uint32_t c = it.chunk;
     const Chunk ch = a.plan.chunks[c];
-    if (meta[kPlanFault] || c >= meta[kChunkCount]) return;
     const uint32_t lane = threadIdx.x & 63, wv = threadIdx.x >> 6, cb = it.column * 4 + wv;
+    // The row table's entries this lane may need (tile wv when the chunk runs as four tiles, tiles 2wv and
+    // 2wv+1 as eight), asked for beside the record: the table covers the whole grid.
+    const int32_t* xr = a.xrows + size_t(c) * 128 + (lane & 15);
+    const int32_t token4 = xr[wv * 16], token8[2] = {xr[(2 * wv) * 16], xr[(2 * wv + 1) * 16]};
+    if (meta[kPlanFault] || c >= meta[kChunkCount]) return;
     const int32_t expert = ch.expert;
     if (expert < 0 || expert >= int32_t(kExperts) || ch.groups < 1 || ch.groups > 8) {
         if (lane == 0) atomicOr(&meta[kFc1Fault], 2u);
@@ -481,8 +484,8 @@ __global__ void __launch_bounds__(kTileThreads, 2) fc1_tile_kernel(Fc1Args a) {
     }
     if (ch.groups == 1) fc1_body<1>(a, ch, cb, lane);
     else if (ch.groups == 2) fc1_body<2>(a, ch, cb, lane);
-    else if (ch.groups <= 4) fc1_tile_body<4>(a, ch, c, cb, wv, lane, lds);
-    else fc1_tile_body<8>(a, ch, c, cb, wv, lane, lds);
+    else if (ch.groups <= 4) fc1_tile_body<4>(a, ch, c, cb, wv, lane, lds, {token4});
+    else fc1_tile_body<8>(a, ch, c, cb, wv, lane, lds, token8);
 }
 
 // 256 threads, one workgroup per (chunk, 256 output columns).
@@ -492,8 +495,9 @@ __global__ void __launch_bounds__(kTileThreads, 2) fc2_tile_kernel(Fc2Args a) {
     const TileItem it = tile_item(kHidden / 256);
     const uint32_t c = it.chunk;
     const Chunk ch = a.plan.chunks[c];
-    if (meta[kPlanFault] || meta[kFc1Fault] || meta[kQuantFault] || c >= meta[kChunkCount]) return;
     const uint32_t lane = threadIdx.x & 63, wv = threadIdx.x >> 6, ob = it.column * 4 + wv;
+    const uint32_t verdict = a.rowbad[c * 16 + (lane & 15)];  // beside the record: the table covers the whole grid
+    if (meta[kPlanFault] || meta[kFc1Fault] || meta[kQuantFault] || c >= meta[kChunkCount]) return;
     const int32_t expert = ch.expert;
     if (expert < 0 || expert >= int32_t(kExperts) || ch.groups < 1 || ch.groups > 8) {
         if (lane == 0) atomicOr(&meta[kFc2Fault], 2u);
@@ -502,8 +506,8 @@ __global__ void __launch_bounds__(kTileThreads, 2) fc2_tile_kernel(Fc2Args a) {
     if (a.skip_from && ch.groups >= a.skip_from) return;  // the stream kernel's share
     if (ch.groups == 1) fc2_body<1>(a, ch, ob, lane);
     else if (ch.groups == 2) fc2_body<2>(a, ch, ob, lane);
-    else if (ch.groups <= 4) fc2_tile_body<4>(a, ch, c, ob, wv, lane, lds);
-    else fc2_tile_body<8>(a, ch, c, ob, wv, lane, lds);
+    else if (ch.groups <= 4) fc2_tile_body<4>(a, ch, c, ob, wv, lane, lds, verdict);
+    else fc2_tile_body<8>(a, ch, c, ob, wv, lane, lds, verdict);
 }
 
 }  // namespace m26g
