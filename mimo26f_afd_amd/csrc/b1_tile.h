@@ -462,6 +462,19 @@ __host__ inline uint32_t tile_grid(uint32_t columns, uint32_t chunk_cap) {
     return columns * ((chunk_cap + 8 * kTileRun - 1) / (8 * kTileRun) * (8 * kTileRun));
 }
 
+// A workgroup's chunk record and the eight meta words, by scalar loads: both are the same for every lane
+// and were written by earlier launches, and the scalar path does not queue behind the operand stream of
+// the workgroup next door, where a vector load of sixteen bytes waits some thousand cycles.
+struct ItemHead { Chunk ch; uint32_t meta[kMetaWords]; };
+__device__ __forceinline__ ItemHead load_item_head(const Chunk* record, const uint32_t* meta) {
+    v4i r;
+    v8i m;
+    asm volatile("s_load_dwordx4 %0, %2, 0x0\n\ts_load_dwordx8 %1, %3, 0x0\n\ts_waitcnt lgkmcnt(0)"
+                 : "=&s"(r), "=&s"(m) : "s"(record), "s"(meta) : "memory");
+    return ItemHead{Chunk{r.x, r.y, r.z, r.w},
+                    {uint32_t(m[0]), uint32_t(m[1]), uint32_t(m[2]), uint32_t(m[3]), uint32_t(m[4]), uint32_t(m[5]), uint32_t(m[6]), uint32_t(m[7])}};
+}
+
 // 256 threads, one workgroup per (chunk, 128 intermediate columns). Chunks of one or two groups run
 // the register-only bodies (each wave is independent there); larger chunks share activations
 // through LDS.
@@ -470,13 +483,14 @@ __global__ void __launch_bounds__(kTileThreads, 2) fc1_tile_kernel(Fc1Args a) {
     uint32_t* meta = a.plan.meta;
     const TileItem it = tile_item(a.lay.inter / 128);
     const uint32_t c = it.chunk;
-    const Chunk ch = a.plan.chunks[c];
     const uint32_t lane = threadIdx.x & 63, wv = threadIdx.x >> 6, cb = it.column * 4 + wv;
     // The row table's entries this lane may need (tile wv when the chunk runs as four tiles, tiles 2wv and
     // 2wv+1 as eight), asked for beside the record: the table covers the whole grid.
     const int32_t* xr = a.xrows + size_t(c) * 128 + (lane & 15);
     const int32_t token4 = xr[wv * 16], token8[2] = {xr[(2 * wv) * 16], xr[(2 * wv + 1) * 16]};
-    if (meta[kPlanFault] || c >= meta[kChunkCount]) return;
+    const ItemHead head = load_item_head(a.plan.chunks + c, meta);  // the chunk table covers the whole grid too
+    const Chunk ch = head.ch;
+    if (head.meta[kPlanFault] || c >= head.meta[kChunkCount]) return;
     const int32_t expert = ch.expert;
     if (expert < 0 || expert >= int32_t(kExperts) || ch.groups < 1 || ch.groups > 8) {
         if (lane == 0) atomicOr(&meta[kFc1Fault], 2u);
@@ -494,10 +508,11 @@ __global__ void __launch_bounds__(kTileThreads, 2) fc2_tile_kernel(Fc2Args a) {
     uint32_t* meta = a.plan.meta;
     const TileItem it = tile_item(kHidden / 256);
     const uint32_t c = it.chunk;
-    const Chunk ch = a.plan.chunks[c];
     const uint32_t lane = threadIdx.x & 63, wv = threadIdx.x >> 6, ob = it.column * 4 + wv;
     const uint32_t verdict = a.rowbad[c * 16 + (lane & 15)];  // beside the record: the table covers the whole grid
-    if (meta[kPlanFault] || meta[kFc1Fault] || meta[kQuantFault] || c >= meta[kChunkCount]) return;
+    const ItemHead head = load_item_head(a.plan.chunks + c, meta);
+    const Chunk ch = head.ch;
+    if (head.meta[kPlanFault] || head.meta[kFc1Fault] || head.meta[kQuantFault] || c >= head.meta[kChunkCount]) return;
     const int32_t expert = ch.expert;
     if (expert < 0 || expert >= int32_t(kExperts) || ch.groups < 1 || ch.groups > 8) {
         if (lane == 0) atomicOr(&meta[kFc2Fault], 2u);
