@@ -815,6 +815,19 @@ __device__ __forceinline__ void fc1_body(const Fc1Args& a, const Chunk ch, uint3
     fc1_finish<TT>(a, ch, cb, lane, acc, bad, live);
 }
 
+// A workgroup's chunk record and the eight meta words, by scalar loads: both are the same for every lane
+// and were written by earlier launches, and the scalar path does not queue behind the operand stream of
+// the workgroup next door, where a vector load of sixteen bytes waits some thousand cycles.
+struct ItemHead { Chunk ch; uint32_t meta[kMetaWords]; };
+__device__ __forceinline__ ItemHead load_item_head(const Chunk* record, const uint32_t* meta) {
+    v4i r;
+    v8i m;
+    asm volatile("s_load_dwordx4 %0, %2, 0x0\n\ts_load_dwordx8 %1, %3, 0x0\n\ts_waitcnt lgkmcnt(0)"
+                 : "=&s"(r), "=&s"(m) : "s"(record), "s"(meta) : "memory");
+    return ItemHead{Chunk{r.x, r.y, r.z, r.w},
+                    {uint32_t(m[0]), uint32_t(m[1]), uint32_t(m[2]), uint32_t(m[3]), uint32_t(m[4]), uint32_t(m[5]), uint32_t(m[6]), uint32_t(m[7])}};
+}
+
 // Stages 2+3: gate/up grouped GEMM, SwiGLU and the v1 requantisation of the intermediate.
 // grid (I/128, chunk capacity), 256 threads; each wave owns one 32-column K32 block of the
 // intermediate for every row of its chunk, so a quantizer block never leaves the wave. A chunk
@@ -823,8 +836,9 @@ template <int NT>
 __global__ void __launch_bounds__(256) fc1_kernel(Fc1Args a) {
     uint32_t* meta = a.plan.meta;
     const uint32_t c = blockIdx.y;
-    const Chunk ch = a.plan.chunks[c];  // fetched beside the verdict words, not after them (the table covers the whole grid)
-    if (meta[kPlanFault] || c >= meta[kChunkCount]) return;
+    const ItemHead head = load_item_head(a.plan.chunks + c, meta);  // the chunk table covers the whole grid
+    const Chunk ch = head.ch;
+    if (head.meta[kPlanFault] || c >= head.meta[kChunkCount]) return;
     const uint32_t lane = threadIdx.x & 63, cb = blockIdx.x * 4 + (threadIdx.x >> 6);
     const int32_t expert = ch.expert;
     if (expert < 0 || expert >= int32_t(kExperts) || ch.groups < 1 || ch.groups > NT) {
@@ -907,8 +921,9 @@ template <int NT>
 __global__ void __launch_bounds__(256) fc2_kernel(Fc2Args a) {
     uint32_t* meta = a.plan.meta;
     const uint32_t c = blockIdx.y;
-    const Chunk ch = a.plan.chunks[c];  // fetched beside the verdict words, not after them
-    if (meta[kPlanFault] || meta[kFc1Fault] || meta[kQuantFault] || c >= meta[kChunkCount]) return;
+    const ItemHead head = load_item_head(a.plan.chunks + c, meta);
+    const Chunk ch = head.ch;
+    if (head.meta[kPlanFault] || head.meta[kFc1Fault] || head.meta[kQuantFault] || c >= head.meta[kChunkCount]) return;
     const uint32_t lane = threadIdx.x & 63, ob = blockIdx.x * 4 + (threadIdx.x >> 6);
     const int32_t expert = ch.expert;
     if (expert < 0 || expert >= int32_t(kExperts) || ch.groups < 1 || ch.groups > NT) {

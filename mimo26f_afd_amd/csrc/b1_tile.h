@@ -462,19 +462,6 @@ __host__ inline uint32_t tile_grid(uint32_t columns, uint32_t chunk_cap) {
     return columns * ((chunk_cap + 8 * kTileRun - 1) / (8 * kTileRun) * (8 * kTileRun));
 }
 
-// A workgroup's chunk record and the eight meta words, by scalar loads: both are the same for every lane
-// and were written by earlier launches, and the scalar path does not queue behind the operand stream of
-// the workgroup next door, where a vector load of sixteen bytes waits some thousand cycles.
-struct ItemHead { Chunk ch; uint32_t meta[kMetaWords]; };
-__device__ __forceinline__ ItemHead load_item_head(const Chunk* record, const uint32_t* meta) {
-    v4i r;
-    v8i m;
-    asm volatile("s_load_dwordx4 %0, %2, 0x0\n\ts_load_dwordx8 %1, %3, 0x0\n\ts_waitcnt lgkmcnt(0)"
-                 : "=&s"(r), "=&s"(m) : "s"(record), "s"(meta) : "memory");
-    return ItemHead{Chunk{r.x, r.y, r.z, r.w},
-                    {uint32_t(m[0]), uint32_t(m[1]), uint32_t(m[2]), uint32_t(m[3]), uint32_t(m[4]), uint32_t(m[5]), uint32_t(m[6]), uint32_t(m[7])}};
-}
-
 // 256 threads, one workgroup per (chunk, 128 intermediate columns). Chunks of one or two groups run
 // the register-only bodies (each wave is independent there); larger chunks share activations
 // through LDS.
