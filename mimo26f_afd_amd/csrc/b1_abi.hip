@@ -173,7 +173,7 @@ void launch_ffn(const m26s_b1_layer* L, m26s_b1_scratch* S, const PlanView& pv, 
     (void)hipEventRecord(S->ea, S->st);
     Fc2Args f2{L->prepared, L->lay, pv, S->dq.as<uint8_t>(), S->dqs.as<uint8_t>(), zero, zero + 8192,
                S->y.as<float>(), uint32_t(routes), nullptr, nullptr, nullptr, 0};
-    fc2_kernel<NT><<<dim3(16, chunk_cap), 256, 0, S->st>>>(f2);
+    fc2_kernel<NT><<<dim3(16 / kFc2Blocks, chunk_cap), 256, 0, S->st>>>(f2);
     (void)hipEventRecord(S->ec, S->st);
 }
 

@@ -617,13 +617,21 @@ __device__ __forceinline__ void mfma_step(v4f (&acc)[4][TT], const WeightStep& w
 // times the memory latency asks for. Activation rows come from L2 and run one k-step ahead; the
 // weight scale dwords of the next quad of k-steps are fetched a quad ahead. Past the end the last
 // k-step is fetched again rather than branching.
-template <int TT>
-__device__ __forceinline__ void gemm_chunk(v4f (&acc)[4][TT], const uint8_t* __restrict__ wp,
-                                           const uint8_t* __restrict__ sp, int ksteps,
-                                           const uint8_t* const (&xrow)[TT], const uint8_t* const (&xsrow)[TT],
-                                           uint32_t lane, uint32_t& bad) {
+// `blocks` consecutive weight blocks (their fragments and scale dwords lie back to back) against the
+// same activation rows, one after the other: the weight stream does not restart between them, the
+// accumulators are handed to `done(b)` after block b and cleared. One block is the plain case.
+template <int TT, class Done>
+__device__ __forceinline__ void gemm_blocks(v4f (&acc)[4][TT], const uint8_t* __restrict__ wp,
+                                            const uint8_t* __restrict__ sp, int ksteps, int blocks,
+                                            const uint8_t* const (&xrow)[TT], const uint8_t* const (&xsrow)[TT],
+                                            uint32_t lane, uint32_t& bad, Done done) {
     const uint32_t shift = 8 * (lane >> 4);
-    const int quads = ksteps / 4, last = ksteps - 1;
+    const int quads = ksteps / 4, last = blocks * ksteps - 1, last_quad = blocks * quads - 1;
+    auto weights_at = [&](int g) { return g < last ? g : last; };
+    auto acts_at = [&](int local, int g) {  // the rows start over with every block; `local` counts inside block b
+        local -= g > last ? g - last : 0;
+        return local >= ksteps ? local - ksteps : local;
+    };
     WeightStep w[4];
     ActStep<TT> x[2];
     uint32_t sw[4], swn[4];
@@ -633,25 +641,39 @@ __device__ __forceinline__ void gemm_chunk(v4f (&acc)[4][TT], const uint8_t* __r
     load_acts<TT>(x[0], 0, xrow, xsrow);
 #pragma unroll
     for (int t = 0; t < 4; ++t) sw[t] = *reinterpret_cast<const uint32_t*>(sp + t * 256);
-    for (int q = 0; q < quads; ++q) {
-        const int ks = 4 * q, qn = q + 1 < quads ? q + 1 : q;
+    for (int b = 0; b < blocks; ++b) {
 #pragma unroll
-        for (int t = 0; t < 4; ++t) swn[t] = *reinterpret_cast<const uint32_t*>(sp + size_t(qn) * 1024 + t * 256);
-        load_weights(w[3], wp, ks + 3);
-        load_acts<TT>(x[1], ks + 1, xrow, xsrow);
-        mfma_step<TT, 0>(acc, w[0], x[0], sw, shift, bad);
-        load_weights(w[0], wp, ks + 4 < last ? ks + 4 : last);
-        load_acts<TT>(x[0], ks + 2, xrow, xsrow);
-        mfma_step<TT, 1>(acc, w[1], x[1], sw, shift, bad);
-        load_weights(w[1], wp, ks + 5 < last ? ks + 5 : last);
-        load_acts<TT>(x[1], ks + 3, xrow, xsrow);
-        mfma_step<TT, 2>(acc, w[2], x[0], sw, shift, bad);
-        load_weights(w[2], wp, ks + 6 < last ? ks + 6 : last);
-        load_acts<TT>(x[0], ks + 4 < last ? ks + 4 : last, xrow, xsrow);
-        mfma_step<TT, 3>(acc, w[3], x[1], sw, shift, bad);
+        for (int t = 0; t < 4; ++t)
 #pragma unroll
-        for (int t = 0; t < 4; ++t) sw[t] = swn[t];
+            for (int tt = 0; tt < TT; ++tt) acc[t][tt] = v4f{0.f, 0.f, 0.f, 0.f};
+        for (int q = 0; q < quads; ++q) {
+            const int g = b * ksteps + 4 * q, gq = b * quads + q, qn = gq < last_quad ? gq + 1 : last_quad;
+#pragma unroll
+            for (int t = 0; t < 4; ++t) swn[t] = *reinterpret_cast<const uint32_t*>(sp + size_t(qn) * 1024 + t * 256);
+            load_weights(w[3], wp, g + 3);
+            load_acts<TT>(x[1], acts_at(4 * q + 1, g + 1), xrow, xsrow);
+            mfma_step<TT, 0>(acc, w[0], x[0], sw, shift, bad);
+            load_weights(w[0], wp, weights_at(g + 4));
+            load_acts<TT>(x[0], acts_at(4 * q + 2, g + 2), xrow, xsrow);
+            mfma_step<TT, 1>(acc, w[1], x[1], sw, shift, bad);
+            load_weights(w[1], wp, weights_at(g + 5));
+            load_acts<TT>(x[1], acts_at(4 * q + 3, g + 3), xrow, xsrow);
+            mfma_step<TT, 2>(acc, w[2], x[0], sw, shift, bad);
+            load_weights(w[2], wp, weights_at(g + 6));
+            load_acts<TT>(x[0], acts_at(4 * q + 4, g + 4), xrow, xsrow);
+            mfma_step<TT, 3>(acc, w[3], x[1], sw, shift, bad);
+#pragma unroll
+            for (int t = 0; t < 4; ++t) sw[t] = swn[t];
+        }
+        done(b);
     }
+}
+template <int TT>
+__device__ __forceinline__ void gemm_chunk(v4f (&acc)[4][TT], const uint8_t* __restrict__ wp,
+                                           const uint8_t* __restrict__ sp, int ksteps,
+                                           const uint8_t* const (&xrow)[TT], const uint8_t* const (&xsrow)[TT],
+                                           uint32_t lane, uint32_t& bad) {
+    gemm_blocks<TT>(acc, wp, sp, ksteps, 1, xrow, xsrow, lane, bad, [](int) {});
 }
 
 // e^t for t <= 0 in binary32: Cody-Waite reduction by ln 2 (two FMAs), the hardware 2^x on the
@@ -884,9 +906,10 @@ __device__ __forceinline__ void fc2_finish(const Fc2Args& a, uint32_t ob, uint32
     if (lost) atomicOr(&a.plan.meta[kFc2Fault], 5u);
 }
 
-// One wave's share of FC2 for a chunk of TT groups: 64 output columns x 16*TT rows.
+// One wave's share of FC2 for a chunk of TT groups: 64 output columns x 16*TT rows per block, `blocks`
+// neighbouring blocks from `ob` on in one uninterrupted weight stream.
 template <int TT>
-__device__ __forceinline__ void fc2_body(const Fc2Args& a, const Chunk ch, uint32_t ob, uint32_t lane) {
+__device__ __forceinline__ void fc2_body(const Fc2Args& a, const Chunk ch, uint32_t ob, uint32_t lane, uint32_t blocks = 1) {
     const uint32_t r = lane & 15, g = lane >> 4, I = a.lay.inter;
     const Group* grp = a.plan.groups + ch.first_group;
     const int32_t expert = ch.expert;
@@ -906,17 +929,17 @@ __device__ __forceinline__ void fc2_body(const Fc2Args& a, const Chunk ch, uint3
     const uint8_t* wp = img + a.lay.w2() + uint64_t(ob) * ksteps * 4096 + lane * 16;
     const uint8_t* sp = img + a.lay.s2() + uint64_t(ob) * (ksteps / 4) * 1024 + lane * 4;
     v4f acc[4][TT];
-#pragma unroll
-    for (int t = 0; t < 4; ++t)
-#pragma unroll
-        for (int tt = 0; tt < TT; ++tt) acc[t][tt] = v4f{0.f, 0.f, 0.f, 0.f};
     uint32_t bad = 0;
-    gemm_chunk<TT>(acc, wp, sp, int(ksteps), xrow, xsrow, lane, bad);
-    fc2_finish<TT>(a, ob, lane, acc, route);
+    gemm_blocks<TT>(acc, wp, sp, int(ksteps), int(blocks), xrow, xsrow, lane, bad,
+                    [&](int b) { fc2_finish<TT>(a, ob + uint32_t(b), lane, acc, route); });
 }
 
 // Stage 4a: down grouped GEMM on the requantised intermediate; rows go back to y[original route].
-// grid (16, chunk capacity), 256 threads; each wave owns 64 output columns.
+// grid (16 / kFc2Blocks, chunk capacity), 256 threads; each wave owns kFc2Blocks x 64 output columns, one
+// block after the other in one weight stream. FC2's stream per block is half as long as FC1's (K = I against
+// K = H), but two blocks per wave halve the workgroups, and at 128 tokens the longer tail of the launch costs
+// more than the longer streams save (172 against 154 us): one block it is.
+constexpr uint32_t kFc2Blocks = 1;
 template <int NT>
 __global__ void __launch_bounds__(256) fc2_kernel(Fc2Args a) {
     uint32_t* meta = a.plan.meta;
@@ -924,16 +947,16 @@ __global__ void __launch_bounds__(256) fc2_kernel(Fc2Args a) {
     const ItemHead head = load_item_head(a.plan.chunks + c, meta);
     const Chunk ch = head.ch;
     if (head.meta[kPlanFault] || head.meta[kFc1Fault] || head.meta[kQuantFault] || c >= head.meta[kChunkCount]) return;
-    const uint32_t lane = threadIdx.x & 63, ob = blockIdx.x * 4 + (threadIdx.x >> 6);
+    const uint32_t lane = threadIdx.x & 63, ob = (blockIdx.x * 4 + (threadIdx.x >> 6)) * kFc2Blocks;
     const int32_t expert = ch.expert;
     if (expert < 0 || expert >= int32_t(kExperts) || ch.groups < 1 || ch.groups > NT) {
         if (lane == 0) atomicOr(&meta[kFc2Fault], 2u);
         return;
     }
-    if (NT == 1 || ch.groups == 1) fc2_body<1>(a, ch, ob, lane);
-    else if (NT == 2 || ch.groups == 2) fc2_body<2>(a, ch, ob, lane);
-    else if (NT >= 4 && ch.groups <= 4) fc2_body<(NT >= 4 ? 4 : 1)>(a, ch, ob, lane);
-    else fc2_body<(NT >= 8 ? 8 : 1)>(a, ch, ob, lane);
+    if (NT == 1 || ch.groups == 1) fc2_body<1>(a, ch, ob, lane, kFc2Blocks);
+    else if (NT == 2 || ch.groups == 2) fc2_body<2>(a, ch, ob, lane, kFc2Blocks);
+    else if (NT >= 4 && ch.groups <= 4) fc2_body<(NT >= 4 ? 4 : 1)>(a, ch, ob, lane, kFc2Blocks);
+    else fc2_body<(NT >= 8 ? 8 : 1)>(a, ch, ob, lane, kFc2Blocks);
 }
 
 // Stage 4b: router-weighted combine. Per (token, column): v = 0; for slot 0..7:
