@@ -23,15 +23,35 @@ sys.path.insert(0, os.path.join(ROOT, "oracle"))
 
 HBM_PEAK_GBS = 8000.0           # MI355X HBM3E, published
 MFMA_FP8_PEAK_TFLOPS = 5000.0   # dense FP8 (an FP8 x FP4 block-scaled MFMA issues at the FP8 rate)
-# HBM bytes per launch of the dominant kernels on these workloads, from two rocprofv3 --pmc runs of this
-# file (FETCH_SIZE, WRITE_SIZE), each scaled by what the same counter reads for --copy-probe's 1 GiB copy:
-# one FETCH_SIZE count = 2.0 KiB, one WRITE_SIZE count = 1.0 KiB.
-FC1_DECODE_TRAFFIC_BYTES = int((2.0 * 857916 + 1.0 * 2570) * 1024)
-FC1_PREFILL_TRAFFIC_BYTES = int((2.0 * 2332868 + 1.0 * 140311) * 1024)
+# HBM bytes per launch of the dominant kernels come from the committed counter profile (two rocprofv3 --pmc
+# runs of this file, FETCH_SIZE and WRITE_SIZE, each scaled by what the same counter reads for --copy-probe's
+# 1 GiB copy): its `traffic_bytes <kernel> <bytes>` rows are read at run time, so the figure printed is the
+# one the profile holds, or null when the profile is not there.
+TRAFFIC_PROFILE = os.path.join("profiles", "hbm_traffic_decode128_prefill8192.md")
+PREFILL_WARMUP, PREFILL_SAMPLES = 10, 31   # the reference's timing protocol (tests/b1_core/bench_connected.cuh:73-81)
 
 
 def log(*a):
     print(*a, file=sys.stderr, flush=True)
+
+
+def profiled_traffic(kernel: str):
+    """(HBM bytes per launch of `kernel` from the committed counter profile or None, where it was looked for)."""
+    path = os.path.join(ROOT, TRAFFIC_PROFILE)
+    try:
+        with open(path) as f:
+            for line in f:
+                tok = line.split()
+                if len(tok) == 3 and tok[0] == "traffic_bytes" and tok[1] == kernel:
+                    return int(tok[2]), TRAFFIC_PROFILE
+    except OSError:
+        pass
+    return None, TRAFFIC_PROFILE
+
+
+def spread(samples):
+    a = np.asarray(samples, np.float64)
+    return dict(median=float(np.median(a)), min=float(a.min()), max=float(a.max()), samples=int(a.size))
 
 
 def stage(wl, torch, dev):
@@ -78,15 +98,36 @@ def timed_steps(layer, scratch, d, rows, steps, warmup, torch, b1):
     return wall_ms / steps, e0.elapsed_time(e1) / steps
 
 
+def sampled_steps(layer, scratch, d, rows, samples, warmup, torch, b1):
+    """`samples` single steps, each between its own pair of events on the launch stream: per-step ms."""
+    def one():
+        b1.ffn_enqueue(layer, scratch, d["payload"].data_ptr(), 4096, d["scales"].data_ptr(), 128, d["ids"].data_ptr(),
+                       d["weights"].data_ptr(), rows, d["out"].data_ptr(), None)
+    for _ in range(warmup):
+        one()
+    scratch.sync()
+    pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(samples)]
+    for a, b in pairs:
+        a.record()
+        one()
+        b.record()
+    scratch.sync()
+    torch.cuda.synchronize()
+    return [a.elapsed_time(b) for a, b in pairs]
+
+
 def kernel_phases(layer, scratch, d, rows, reps, b1):
-    """Average per-kernel durations from the HIP events the library records on its launch stream."""
-    acc = np.zeros(5)
+    """Per-kernel durations from the HIP events the library records on its launch stream: the average over
+    `reps` calls (what the roofline figures divide by) and the median / min / max of each."""
+    rows_ = []
     for _ in range(reps):
         s = b1.ffn_dev(layer, scratch, d["payload"].data_ptr(), 4096, d["scales"].data_ptr(), 128, d["ids"].data_ptr(),
                        d["weights"].data_ptr(), rows, d["out"].data_ptr(), None)
-        acc += np.array([s.upload_plan_ms, s.phase_ms[0], s.phase_ms[2], s.phase_ms[3], s.gpu_ms])
-    acc /= reps
-    return dict(plan_ms=acc[0], fc1_ms=acc[1], fc2_ms=acc[2], reduce_ms=acc[3], gpu_ms=acc[4])
+        rows_.append([s.upload_plan_ms, s.phase_ms[0], s.phase_ms[2], s.phase_ms[3], s.gpu_ms])
+    a = np.array(rows_)
+    acc = a.mean(axis=0)
+    return dict(plan_ms=acc[0], fc1_ms=acc[1], fc2_ms=acc[2], reduce_ms=acc[3], gpu_ms=acc[4], reps=reps,
+                fc1=spread(a[:, 1]), fc2=spread(a[:, 2]), reduce=spread(a[:, 3]), plan=spread(a[:, 0]))
 
 
 def sample_parity(wl, pools, got_bits, tokens, O):
@@ -101,17 +142,33 @@ def sample_parity(wl, pools, got_bits, tokens, O):
 
 
 def cpu_baseline(wl, pools, tokens, O):
-    """The CPU restatement of the reference's W4A8 expert path on a bounded sample, all host threads."""
+    """The CPU restatement of the reference's expert path on bounded samples of the same workload: the W4A8
+    lattice (the parity rule: FP64 dots, FP32 boundaries, requantised intermediate) on all host threads,
+    which is `value`, the same on one thread, and the reference's E-FP32 twin (FP32 per-MAC accumulation, no
+    intermediate requantisation; crates/mimo26-expert/src/grouped.rs:291-336) on all threads and on one."""
     threads = O.hardware_threads()
-    t0 = time.perf_counter()
-    rc, _, _, _ = O.layer_ffn(pools, wl.payload[tokens], wl.scales[tokens], wl.ids[tokens], wl.weights[tokens], threads=threads)
-    dt = time.perf_counter() - t0
-    return dict(value=len(tokens) / dt, unit="routed tok/s per MoE layer", cores=threads, kind="port",
-                sample=f"{len(tokens)} tokens ({len(tokens) * 8} routes) of the same workload, W4A8 lattice "
-                       f"(FP64 dots, FP32 boundaries), {dt:.1f}s, rc={rc}")
+    few = tokens[:max(1, len(tokens) // 8)]
+
+    def timed(sample, n_threads, efp32):
+        t0 = time.perf_counter()
+        rc = O.layer_ffn(pools, wl.payload[sample], wl.scales[sample], wl.ids[sample], wl.weights[sample],
+                         threads=n_threads, efp32=efp32)[0]
+        dt = time.perf_counter() - t0
+        return dict(value=len(sample) / dt, unit="routed tok/s per MoE layer", cores=n_threads,
+                    sample=f"{len(sample)} tokens ({len(sample) * 8} routes, {np.unique(wl.ids[sample]).size} experts) of the same workload, "
+                           f"{dt:.1f}s, rc={rc}")
+    full = timed(tokens, threads, False)
+    out = dict(value=full["value"], unit=full["unit"], cores=threads, kind="port",
+               sample="W4A8 lattice (FP64 dots, FP32 boundaries, requantised intermediate): " + full["sample"])
+    out["single_thread"] = timed(few, 1, False)
+    out["efp32"] = dict(all_threads=timed(tokens, threads, True), single_thread=timed(few, 1, True),
+                        rule="E-FP32 twin: FP32 activations and per-MAC FP32 accumulation in k order, no intermediate requantisation")
+    return out
 
 
-def run_config(cfg, steps, warmup, torch, dev, b1, synth, O, parity_tokens, cpu_tokens):
+def run_config(cfg, steps, warmup, torch, dev, b1, synth, O, parity_tokens, cpu_tokens, samples=0):
+    """Correctness before and after the timing, as the reference's bench gate does. `samples` > 0 adds the
+    per-step event protocol (that many single steps after `warmup` warm-ups: median / min / max)."""
     wl = synth.make(cfg)
     log(f"[bench] config {cfg}: {wl.name}")
     layer, pools = build_layer(wl, torch, dev, b1)
@@ -120,23 +177,36 @@ def run_config(cfg, steps, warmup, torch, dev, b1, synth, O, parity_tokens, cpu_
     ph = kernel_phases(layer, scratch, d, wl.rows, 3, b1)  # also the first correctness pass
     before = d["out"].cpu().numpy().view(np.uint16).copy()
     wall_ms, ev_ms = timed_steps(layer, scratch, d, wl.rows, steps, warmup, torch, b1)
-    ph = kernel_phases(layer, scratch, d, wl.rows, 10, b1)
+    per_step = spread(sampled_steps(layer, scratch, d, wl.rows, samples, warmup, torch, b1)) if samples else None
+    ph = kernel_phases(layer, scratch, d, wl.rows, PREFILL_SAMPLES, b1)
     after = d["out"].cpu().numpy().view(np.uint16)
     tokens = np.arange(min(parity_tokens, wl.rows))
     par = sample_parity(wl, pools, after, tokens, O)
     par["bitwise_stable_across_timing"] = bool(np.array_equal(before, after))
     cpu = cpu_baseline(wl, pools, np.arange(min(cpu_tokens, wl.rows)), O) if cpu_tokens else None
     touched = int(wl.touched().size)
-    res = dict(wl=wl, ms_per_step=wall_ms, event_ms_per_step=ev_ms, phases=ph, parity=par, cpu=cpu, touched=touched)
+    res = dict(wl=wl, ms_per_step=wall_ms, event_ms_per_step=ev_ms, per_step=per_step, phases=ph, parity=par, cpu=cpu, touched=touched)
     del layer, scratch
     return res
 
 
-def run_stack(args, torch, dev, O):
-    """configs[4]: the routed experts of `--stack` layers resident in HBM; a prefill in 4096-token
-    segments, a 16-token decode step after each; one JSON line of its own."""
+def stack_reference_rows(seed, layer, payload, scales, ids, weights, O, synth):
+    """The CPU rule's BF16 rows for a few tokens of one stack layer, its touched experts regenerated on the host."""
+    pools = []
+    for r in range(4):
+        pool = np.full(synth.EXPERTS * synth.IMAGE_BYTES, 0x22, np.uint8)
+        for e in np.unique(ids):
+            pool[e * synth.IMAGE_BYTES:(e + 1) * synth.IMAGE_BYTES] = synth.expert_image(seed, r, int(e), layer)
+        pools.append(pool)
+    rc, _, bits, _ = O.layer_ffn(pools, payload, scales, ids, weights)
+    return rc, bits
+
+
+def run_stack(layers, tokens, torch, dev, O):
+    """configs[4]: the routed experts of `layers` layers resident in HBM; a prefill in 4096-token
+    segments, a 16-token decode step after each. Returns the JSON object of the run."""
     from mimo26f_afd_amd import stack as S, synth
-    layers, tokens, seg, dec_rows = args.stack, args.stack_tokens, 4096, 16
+    seg, dec_rows = 4096, 16
     segments = tokens // seg
     t0 = time.time()
     st = S.ResidentStack(layers, torch, dev, log=log)
@@ -180,7 +250,7 @@ def run_stack(args, torch, dev, O):
     dec_ms = np.array([a.elapsed_time(b) for a, b in dec_t])
     parity = []
     for (kind, l), (frame, ids, w, got) in sorted(kept.items()):
-        rc, ref = S.reference_rows(st.seed, l, frame[:, :4096].copy(), frame[:, 4096:4224].copy(), ids, w, O)
+        rc, ref = stack_reference_rows(st.seed, l, frame[:, :4096].copy(), frame[:, 4096:4224].copy(), ids, w, O, synth)
         g = (got.astype(np.uint32) << 16).view(np.float32).astype(np.float64)
         r = (ref.astype(np.uint32) << 16).view(np.float32).astype(np.float64)
         parity.append(dict(batch=kind, layer=l, tokens=len(ids), oracle_rc=rc, max_abs_over_max_ref=float(np.max(np.abs(g - r)) / np.max(np.abs(r))),
@@ -211,7 +281,9 @@ def run_stack(args, torch, dev, O):
         "parity": parity,
     }
     st.close()
-    print(json.dumps(line), flush=True)
+    del st
+    torch.cuda.empty_cache()
+    return line
 
 
 def main():
@@ -226,6 +298,7 @@ def main():
                          "size that scales the FETCH_SIZE / WRITE_SIZE counters")
     ap.add_argument("--only-prefill", action="store_true",
                     help="profiling aid: run only the prefill measurement and print its object")
+    ap.add_argument("--no-stack", action="store_true", help="skip the 48-layer resident stack (configs[4]) object")
     ap.add_argument("--stack", type=int, default=0, metavar="LAYERS",
                     help="run configs[4] instead: this many layers' routed experts resident in HBM (48 = the full model, 164 GB)")
     ap.add_argument("--stack-tokens", type=int, default=65536, help="prefill length of the --stack run (a multiple of 4096)")
@@ -242,7 +315,7 @@ def main():
     torch.cuda.set_device(dev)
 
     if args.stack:
-        run_stack(args, torch, dev, O)
+        print(json.dumps(run_stack(args.stack, args.stack_tokens, torch, dev, O)), flush=True)
         return
     if args.copy_probe:
         src = torch.zeros(1 << 28, dtype=torch.int32, device=dev)
@@ -257,7 +330,7 @@ def main():
         print(json.dumps(dict(ms_per_step=pre["ms_per_step"], phases=pre["phases"], parity=pre["parity"])), flush=True)
         return
     dec = run_config(2, args.steps, args.warmup, torch, dev, b1, synth, O, parity_tokens=8,
-                     cpu_tokens=0 if args.no_cpu else 128)
+                     cpu_tokens=0 if args.no_cpu else 128, samples=PREFILL_SAMPLES)
     wl = dec["wl"]
     inter, U = wl.intermediate, dec["touched"]
     # Algorithmic bytes: unique weight bytes of the touched experts + input rows + ids/weights + BF16 rows;
@@ -266,6 +339,7 @@ def main():
     fc1_bytes = U * inter * (4096 + 256) + wl.rows * 4224
     fc1_gbs = fc1_bytes / (dec["phases"]["fc1_ms"] * 1e-3) / 1e9
     path_gbs = path_bytes / (dec["ms_per_step"] * 1e-3) / 1e9
+    dec_traffic, traffic_source = profiled_traffic("fc1_kernel<2>")
     line = {
         "metric": "routed tok/s per MoE layer; HBM GB/s (decode) and MFMA % of peak (prefill)",
         "value": wl.rows / (dec["ms_per_step"] * 1e-3),
@@ -278,10 +352,12 @@ def main():
                    "activations": "bf16 N(0,1) -> wire quantizer FP8 e4m3 + ue8m0/32"},
         "roofline": {"bound": "hbm", "kernel": "fc1_kernel<2> (gate/up GEMM + SwiGLU + requant)",
                      "achieved": fc1_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": fc1_gbs / HBM_PEAK_GBS,
-                     "traffic": FC1_DECODE_TRAFFIC_BYTES, "algorithmic_bytes": fc1_bytes, "kernel_ms": dec["phases"]["fc1_ms"],
+                     "traffic": dec_traffic, "traffic_source": traffic_source, "algorithmic_bytes": fc1_bytes,
+                     "kernel_ms": dec["phases"]["fc1_ms"], "kernel_ms_spread": dec["phases"]["fc1"],
                      "path": {"algorithmic_bytes": path_bytes, "achieved": path_gbs, "frac": path_gbs / HBM_PEAK_GBS,
                               "plan_ms": dec["phases"]["plan_ms"], "fc2_ms": dec["phases"]["fc2_ms"],
-                              "reduce_ms": dec["phases"]["reduce_ms"], "event_ms_per_step": dec["event_ms_per_step"]}},
+                              "reduce_ms": dec["phases"]["reduce_ms"], "event_ms_per_step": dec["event_ms_per_step"],
+                              "fc2_ms_spread": dec["phases"]["fc2"], "per_step_ms": dec["per_step"]}},
         "cpu_baseline": dec["cpu"],
         "parity": dec["parity"],
     }
@@ -293,29 +369,49 @@ def main():
     line["roofline"]["path"]["frac_of_measured"] = path_gbs / read_gbs
     line["value_routes_per_s"] = line["value"] * 8
     if not args.no_prefill:
-        pre = run_config(3, max(3, args.steps // 5), max(2, args.warmup // 5), torch, dev, b1, synth, O, parity_tokens=4,
-                         cpu_tokens=0)
+        # The reference's protocol: at least 10 warm-ups, at least 31 single-step event samples, the median reported.
+        p_warm, p_samples = max(PREFILL_WARMUP, args.warmup), max(PREFILL_SAMPLES, args.steps)
+        pre = run_config(3, p_samples, p_warm, torch, dev, b1, synth, O, parity_tokens=4, cpu_tokens=0, samples=p_samples)
         pw = pre["wl"]
         flops = pw.flops()
-        tf = flops / (pre["ms_per_step"] * 1e-3) / 1e12
+        step_ms = pre["per_step"]["median"]
+        tf = flops / (step_ms * 1e-3) / 1e12
         fc1_flops = 4 * pw.rows * 8 * 4096 * pw.intermediate
-        fc1_tf = fc1_flops / (pre["phases"]["fc1_ms"] * 1e-3) / 1e12
+        fc1_ms = pre["phases"]["fc1"]["median"]
+        fc1_tf = fc1_flops / (fc1_ms * 1e-3) / 1e12
+        pre_traffic, _ = profiled_traffic("fc1_tile_kernel")
         line["prefill"] = {
             "workload": "configs[3]: one full MoE layer, prefill chunk, 8192 tokens, Zipf(1.1) routing",
-            "value": pw.rows / (pre["ms_per_step"] * 1e-3), "unit": "routed tok/s per MoE layer",
-            "ms_per_step": pre["ms_per_step"], "steps": max(3, args.steps // 5),
+            "value": pw.rows / (step_ms * 1e-3), "unit": "routed tok/s per MoE layer",
+            "ms_per_step": step_ms, "ms_per_step_spread": pre["per_step"], "warmup": p_warm,
+            "ms_per_step_back_to_back": pre["ms_per_step"], "steps": p_samples,
             "roofline": {"bound": "mfma", "kernel": "fc1_tile_kernel (gate/up GEMM + SwiGLU + requant)", "achieved": fc1_tf, "peak": MFMA_FP8_PEAK_TFLOPS,
-                         "unit": "TFLOP/s", "frac": fc1_tf / MFMA_FP8_PEAK_TFLOPS, "traffic": FC1_PREFILL_TRAFFIC_BYTES,
-                         "algorithmic_flops": fc1_flops, "kernel_ms": pre["phases"]["fc1_ms"],
+                         "unit": "TFLOP/s", "frac": fc1_tf / MFMA_FP8_PEAK_TFLOPS, "traffic": pre_traffic, "traffic_source": traffic_source,
+                         "algorithmic_flops": fc1_flops, "kernel_ms": fc1_ms, "kernel_ms_spread": pre["phases"]["fc1"],
                          "path": {"algorithmic_flops": flops, "achieved": tf, "frac": tf / MFMA_FP8_PEAK_TFLOPS,
-                                  "plan_ms": pre["phases"]["plan_ms"], "fc2_ms": pre["phases"]["fc2_ms"],
-                                  "reduce_ms": pre["phases"]["reduce_ms"]}},
+                                  "plan_ms": pre["phases"]["plan"]["median"], "fc2_ms": pre["phases"]["fc2"]["median"],
+                                  "reduce_ms": pre["phases"]["reduce"]["median"], "fc2_ms_spread": pre["phases"]["fc2"]}},
             "parity": pre["parity"],
         }
         mfma_tf = probe.mfma_rate_tflops()
         line["prefill"]["roofline"]["measured_mfma_TFLOPs"] = mfma_tf
         line["prefill"]["roofline"]["frac_of_measured"] = fc1_tf / mfma_tf
         line["prefill"]["roofline"]["path"]["frac_of_measured"] = tf / mfma_tf
+    if not args.no_stack:
+        # configs[4] with all 48 layers resident needs about 175 GiB of HBM; without it the object says so.
+        free_gib = torch.cuda.mem_get_info()[0] / 2**30
+        if free_gib < 200:
+            line["stack"] = {"skipped": f"{free_gib:.0f} GiB of HBM free, the 48-layer stack holds 175"}
+        else:
+            try:
+                t0 = time.time()
+                st = run_stack(48, 65536, torch, dev, O)
+                line["stack"] = {"workload": st["config"]["workload"], "value": st["value"], "unit": st["unit"],
+                                 "whole_schedule_ms": st["config"]["whole_schedule_ms"], "hbm_held_GiB": st["config"]["hbm_held_GiB"],
+                                 "prefill_ffn": st["prefill_ffn"], "decode_ffn": st["decode_ffn"], "parity": st["parity"],
+                                 "leg_seconds": time.time() - t0}
+            except Exception as e:  # the headline line must survive a failure of this leg
+                line["stack"] = {"error": f"{type(e).__name__}: {e}"}
     print(json.dumps(line), flush=True)
 
 

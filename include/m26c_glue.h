@@ -43,8 +43,9 @@ int m26c_quantize_hidden(const float* x, long rows, int cols, uint8_t* payload, 
 
 /* crates/mimo26-coordinator/kernels/glue.cu:309-348. Writes the request frame's route entries
  * (12 bytes each: row u32, expert u32, weight f32 bits; t * topk of them) and its hidden rows (hid
- * payload bytes then hid / 32 scale bytes, at `pitch`). hid must be a multiple of 256; routes 4-byte and
- * hidden 8-byte aligned, pitch a multiple of 8. */
+ * payload bytes then hid / 32 scale bytes, at `pitch`). hid must be a multiple of 256; payload 16-byte,
+ * scales and hidden 8-byte and routes 4-byte aligned, pitch a multiple of 8 (a request frame's hidden rows
+ * start on 8-byte boundaries only); anything else returns 1. */
 int m26c_frame_fill(const int* idx, const float* wts, const uint8_t* payload, const uint8_t* scales, int t, int topk,
                     int hid, uint8_t* routes, uint8_t* hidden, int pitch, void* stream);
 

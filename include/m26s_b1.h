@@ -32,7 +32,11 @@ typedef struct m26s_b1_scratch m26s_b1_scratch;
  * keeps its own permuted copy; the caller may free canonical_dev on return. */
 int m26s_b1_layer_new(const uint8_t* canonical_dev, uint64_t canonical_bytes, uint32_t rank,
                       m26s_b1_layer** out, char* err, size_t errlen);
-/* b1_serve.cu:268. 1 when every weight scale byte lies in [2, 252]. */
+/* b1_serve.cu:268. 1 when every weight scale byte lies in [2, 252]. A layer for which this is 0 is
+ * served all the same: its calls take the conforming arm (each weight decoded by the format's rule,
+ * min(s, 254) and saturation at +-FLT_MAX included, then multiplied; the counterpart of the reference's
+ * decode-then-fmaf arm, crates/mimo26-expert/kernels/b1/grouped.cu:42-67), far slower than the matrix
+ * pipe. Real checkpoints hold scale bytes 118..125 and never take it. */
 int m26s_b1_layer_all_normal(const m26s_b1_layer* layer);
 /* b1_serve.cu:270-276. */
 void m26s_b1_layer_free(m26s_b1_layer* layer);
@@ -77,6 +81,10 @@ int m26s_b1_layer_view(const m26s_b1_layer* layer, const uint8_t** prepared_dev,
  * default stream) instead of creating its own, so the caller can bracket calls with its own
  * events. The stream is not owned. */
 int m26s_b1_scratch_new_on(void* hip_stream, m26s_b1_scratch** out, char* err, size_t errlen);
+/* The hipStream_t (as void*) the scratch launches on, its own or the caller's: whoever writes the
+ * inputs of an enqueued call on the device has to order those writes before the call, which work on
+ * this stream is and work on another stream is not. */
+void* m26s_b1_scratch_stream(const m26s_b1_scratch* scratch);
 
 /* m26s_b1_ffn with DEVICE pointers for every array: no PCIe in the call. payload_dev must be
  * 16-byte aligned with payload_pitch % 16 == 0; scales_dev 4-byte aligned with
@@ -87,7 +95,9 @@ int m26s_b1_ffn_dev(const m26s_b1_layer* layer, m26s_b1_scratch* scratch, const 
                     const int32_t* ids_dev, const float* weights_dev, uint32_t rows,
                     uint16_t* bf16_out_dev, float* partial_dev, float* ms, char* err, size_t errlen);
 /* Same work, enqueued only: returns after the launches. Faults of every call since the last
- * m26s_b1_scratch_sync accumulate and are reported there. */
+ * m26s_b1_scratch_sync accumulate and are reported there: once a call's routes have been rejected or
+ * one of its stages has faulted, the later calls enqueued on the scratch before that sync compute
+ * nothing, and the sync returns the first fault's code (3 before 4). */
 int m26s_b1_ffn_enqueue(const m26s_b1_layer* layer, m26s_b1_scratch* scratch, const uint8_t* payload_dev,
                         size_t payload_pitch, const uint8_t* scales_dev, size_t scales_pitch,
                         const int32_t* ids_dev, const float* weights_dev, uint32_t rows,
@@ -118,15 +128,6 @@ int m26s_b1_reduce_dev(const float* y_dev, const float* weights_dev, uint32_t ro
 
 /* With taps on, the next FFN calls also keep FP32 gate / up / h of every grouped row. */
 void m26s_b1_scratch_set_taps(m26s_b1_scratch* scratch, int on);
-/* No counterpart in the reference. Off by default. When on, prefill-size calls (more than 128 rows) on
- * a full-intermediate layer run FC2's chunks of five to eight groups through one persistent
- * eight-wave workgroup per compute unit (operands in one pipeline across work items, the finished
- * accumulators stored under the next item's MFMAs) and leave the smaller chunks to the tile kernel.
- * Results are bit for bit those of the default schedule; at 8192 tokens it is measured slower
- * (0.85 against 0.75 ms: FC2 is bound by the writes of the per-route rows either way, and the small
- * chunks no longer overlap the large ones), so it is kept as the tested base of the FC1 kernel of the
- * same shape, not as the serving path. */
-void m26s_b1_scratch_set_stream(m26s_b1_scratch* scratch, int on);
 /* Device address and byte size of an internal buffer after a call. which: 0 inverse, 1 original
  * routes, 2 grouped weights, 3 groups, 4 meta words {group count, plan fault, chunk count, fc1
  * fault, quantizer fault, lowest faulting block, fc2 fault, reduce fault}, 5 intermediate payload

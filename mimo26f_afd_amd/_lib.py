@@ -9,13 +9,11 @@ from . import build
 _u8p, _f32p, _i32p, _u32p, _u16p = (C.POINTER(t) for t in (C.c_uint8, C.c_float, C.c_int32, C.c_uint32, C.c_uint16))
 _vp, _sz, _cp = C.c_void_p, C.c_size_t, C.c_char_p
 
-# name -> (restype, argtypes); every symbol include/m26s_b1.h, include/m26c_glue.h, include/m26_probe.h and include/m26w_frame.h declare
+# name -> (restype, argtypes); every symbol include/m26s_b1.h, include/m26c_glue.h and include/m26w_frame.h declare
 SIGNATURES = {
     "m26w_crc32c_update": (C.c_uint32, [C.c_uint32, _vp, _sz]),
     "m26w_request_routes_dev": (C.c_int, [_vp, _vp, C.c_uint32, C.c_uint32, _vp, _vp, _vp, _vp]),
     "m26w_stage_rows_dev": (C.c_int, [_vp, _vp, _sz, _vp]),
-    "m26p_read_bandwidth": (C.c_int, [C.c_uint64, C.c_int, _vp, C.POINTER(C.c_double), _cp, _sz]),
-    "m26p_mfma_rate": (C.c_int, [C.c_int, C.c_int, _vp, C.POINTER(C.c_double), _cp, _sz]),
     "m26c_router_topk": (C.c_int, [_vp, _vp, C.c_int, C.c_int, C.c_int, _vp, _vp, _vp]),
     "m26c_quant_scales": (C.c_int, [_vp, C.c_long, _vp, _vp, _vp]),
     "m26_quantize_hidden_fp8": (C.c_int, [_vp, _vp, _vp, C.c_int64, _vp]),
@@ -41,7 +39,7 @@ SIGNATURES = {
     "m26s_b1_quantize_dev": (C.c_int, [_vp, C.c_uint64, _vp, _vp, _vp, _cp, _sz]),
     "m26s_b1_reduce_dev": (C.c_int, [_vp, _vp, C.c_uint32, _vp, _vp, _vp, _cp, _sz]),
     "m26s_b1_scratch_set_taps": (None, [_vp, C.c_int]),
-    "m26s_b1_scratch_set_stream": (None, [_vp, C.c_int]),
+    "m26s_b1_scratch_stream": (_vp, [_vp]),
     "m26s_b1_scratch_view": (C.c_int, [_vp, C.c_int, C.POINTER(_vp), C.POINTER(_sz)]),
     "m26s_b1_copy_to_host": (C.c_int, [_vp, _vp, _sz]),
     "m26s_b1_copy_to_device": (C.c_int, [_vp, _vp, _sz]),
@@ -49,20 +47,47 @@ SIGNATURES = {
     "m26s_b1_device_free": (None, [_vp]),
 }
 
+# the measurement library's symbols (include/m26_probe.h)
+PROBE_SIGNATURES = {
+    "m26p_read_bandwidth": (C.c_int, [C.c_uint64, C.c_int, _vp, C.POINTER(C.c_double), _cp, _sz]),
+    "m26p_mfma_rate": (C.c_int, [C.c_int, C.c_int, _vp, C.POINTER(C.c_double), _cp, _sz]),
+}
+
 _LIB = None
+_PROBE = None
+
+
+def _bind(path: str, signatures: dict) -> C.CDLL:
+    lib = C.CDLL(path)
+    for name, (res, args) in signatures.items():
+        fn = getattr(lib, name)  # AttributeError here = a declared symbol is not exported
+        fn.restype = res
+        fn.argtypes = args
+    return lib
+
+
+def _on_gpu_box() -> bool:
+    return os.path.exists("/dev/kfd")
 
 
 def load() -> C.CDLL:
-    """The built library; built first only if nothing is there."""
+    """The built serving library. It is built here only if nothing is there, or, on a machine without a
+    GPU (where libraries are built, not run), if a source is newer than it: a GPU run loads what it was
+    handed and never compiles."""
     global _LIB
     if _LIB is None:
         path = os.environ.get("M26S_B1_LIB") or build.LIB  # a deployment may point at its own build
-        if path == build.LIB and not os.path.exists(path):
+        if path == build.LIB and (not os.path.exists(path) or (build.stale() and not _on_gpu_box())):
             build.build_library()
-        lib = C.CDLL(path)
-        for name, (res, args) in SIGNATURES.items():
-            fn = getattr(lib, name)  # AttributeError here = a declared symbol is not exported
-            fn.restype = res
-            fn.argtypes = args
-        _LIB = lib
+        _LIB = _bind(path, SIGNATURES)
     return _LIB
+
+
+def load_probe() -> C.CDLL:
+    """The measurement library (roofline probes), built on the same terms."""
+    global _PROBE
+    if _PROBE is None:
+        if not os.path.exists(build.PROBE_LIB) or (build.probe_stale() and not _on_gpu_box()):
+            build.build_probe()
+        _PROBE = _bind(build.PROBE_LIB, PROBE_SIGNATURES)
+    return _PROBE

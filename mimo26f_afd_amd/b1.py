@@ -106,9 +106,10 @@ class Scratch:
     def set_taps(self, on: bool) -> None:
         load().m26s_b1_scratch_set_taps(self._h, 1 if on else 0)
 
-    def set_stream(self, on: bool) -> None:
-        """FC2's large chunks through the persistent kernel (off by default; same bits, measured slower)."""
-        load().m26s_b1_scratch_set_stream(self._h, 1 if on else 0)
+    @property
+    def stream(self) -> int:
+        """The HIP stream the scratch launches on (0 for the default stream)."""
+        return int(load().m26s_b1_scratch_stream(self._h) or 0)
 
     def sync(self) -> None:
         buf = _err()

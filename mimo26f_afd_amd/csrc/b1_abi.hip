@@ -1,46 +1,53 @@
-// C ABI of the gfx950 routed-expert FFN: handles, buffer ownership, launch schedule, fault decode.
-// Mirrors the contract of crates/mimo26-spark/kernels/b1_serve.cu:145-574 of the reference (names,
-// argument meaning, return codes, the ms[8] phase report); the schedule itself is new: no host
-// round trip between the planner and the GEMMs (grids are sized by capacity and idle workgroups
-// leave on the device-side counts), and the intermediate quantizer is fused into FC1.
+// C ABI of the gfx950 routed-expert FFN: handles, the per-call workspace, launch schedule, fault decode.
+// Keeps the contract of crates/mimo26-spark/kernels/b1_serve.cu:214-574 of the reference (names,
+// argument meaning, return codes, the ms[8] phase report). What is behind it is this library's own:
+// every per-call array is carved out of one grow-only slab by a layout function of (rows, intermediate),
+// there is no host round trip between the planner and the GEMMs (grids are sized by capacity and idle
+// workgroups leave on the device-side counts), the intermediate quantizer is fused into FC1, and a
+// layer with exceptional weight scales runs the conforming arm of b1_conform.h.
 #include <hip/hip_runtime.h>
 #include <chrono>
+#include <cstdarg>
 #include <cstdio>
 #include <cstring>
 #include <new>
 #include <vector>
 
 #include "../../include/m26s_b1.h"
-#include "b1_stream.h"
+#include "b1_conform.h"
+#include "b1_tile.h"
 
 using namespace m26g;
 
 namespace {
 
-struct Dev {
-    void* p = nullptr;
-    size_t n = 0;
-    hipError_t ensure(size_t bytes) {
-        if (bytes <= n) return hipSuccess;
-        if (p) (void)hipFree(p);
-        p = nullptr;
-        n = 0;
-        const size_t want = bytes < 256 ? 256 : bytes;
-        const hipError_t e = hipMalloc(&p, want);
-        if (e == hipSuccess) n = want;
-        return e;
+// ---- the error channel of one call ------------------------------------------------------------------
+// The first failure of a call decides its return code and its message; `text` is the caller's buffer.
+class Outcome {
+public:
+    Outcome(char* text, size_t room) : text_(text), room_(room) {}
+    int fail(int rc, const char* fmt, ...) __attribute__((format(printf, 3, 4))) {
+        if (text_ && room_) {
+            va_list ap;
+            va_start(ap, fmt);
+            std::vsnprintf(text_, room_, fmt, ap);
+            va_end(ap);
+        }
+        return rc;
     }
-    template <class T> T* as() const { return static_cast<T*>(p); }
-    ~Dev() { if (p) (void)hipFree(p); }
+    // 0 when the runtime call succeeded, else return code 2 with "<step>: <runtime message>".
+    int runtime(hipError_t e, const char* step) { return e == hipSuccess ? 0 : fail(2, "%s: %s", step, hipGetErrorString(e)); }
+
+private:
+    char* text_;
+    size_t room_;
 };
+#define M26G_TRY(out, call, step)                         \
+    do {                                                  \
+        if (const int rc_ = (out).runtime((call), step)) return rc_; \
+    } while (0)
 
-void set_err(char* err, size_t len, const char* what, hipError_t e) {
-    if (err && len) std::snprintf(err, len, "%s: %s", what, hipGetErrorString(e));
-}
-void set_msg(char* err, size_t len, const char* msg) {
-    if (err && len) std::snprintf(err, len, "%s", msg);
-}
-
+// ---- sizes ---------------------------------------------------------------------------------------------
 uint32_t capacity_class(uint32_t rows) { return rows <= 256 ? 256u : rows <= 2048 ? 2048u : rows <= 4096 ? 4096u : 8192u; }
 // Groups of at most 16 rows: every expert adds at most one ragged group.
 uint64_t group_bound(uint64_t routes) { const uint64_t b = routes / 16 + kExperts; return b < routes ? b : routes; }
@@ -55,10 +62,104 @@ uint64_t chunk_bound(uint64_t routes, uint32_t gpc) {
 constexpr uint32_t kWidePlanFrom = 512;  // rows above which the planner runs on several compute units
 uint32_t tiles_for(uint32_t rows) { return rows <= 32 ? 1u : rows <= 128 ? 2u : 8u; }
 
+// ---- the workspace of one call --------------------------------------------------------------------------
+// Everything a call needs beyond its inputs and outputs, as pointers into one slab. `Fixed` survives from
+// call to call (the fault words accumulate until the next sync; the zero row and the unit scales are
+// written once); the rest is per call and may move when the slab grows.
+struct Fixed {
+    uint32_t* meta;      // kMetaWords fault / count words
+    uint8_t* zero_row;   // 8192 zero bytes: the activation row of a padded tile row
+    uint8_t* unit_scales;  // 256 bytes of 127
+};
+constexpr size_t kFixedBytes = 256 + 8192 + 256;
+Fixed fixed_at(uint8_t* base) {
+    return Fixed{reinterpret_cast<uint32_t*>(base), base + 256, base + 256 + 8192};
+}
+__global__ void fixed_init_kernel(uint8_t* base) {  // a kernel, not a memset: a caller may be recording a graph
+    for (uint32_t i = threadIdx.x; i < kFixedBytes; i += blockDim.x)  // meta word kQuantWhere starts at "no block"
+        base[i] = i >= 256 + 8192 ? uint8_t(127) : (i / 4 == kQuantWhere ? uint8_t(0xff) : uint8_t(0));
+}
+
+struct Shape {
+    uint32_t rows, inter;
+    bool taps, host_io, conforming;
+};
+struct Workspace {
+    uint32_t* plan_work;  // the wide planner's histograms (always first: its header word is armed when the slab moves)
+    int32_t *inverse, *original;
+    float* grouped_weights;
+    Group* groups;
+    Chunk* chunks;
+    uint8_t *dq, *dqs;
+    float* y;
+    uint8_t *xg, *dg;  // tile schedule: activation scales in MFMA lane order
+    uint32_t* rowbad;
+    int32_t *xrows, *yrows;
+    float *tap_gate, *tap_up, *tap_h;
+    uint8_t *x, *xs;  // host entry: staged inputs and output
+    int32_t* ids;
+    float* weights;
+    uint16_t* bf16;
+    size_t bytes[20];  // extents of the views m26s_b1_scratch_view hands out, by its `which`
+    size_t total;
+    uint32_t tiles, chunk_cap, group_cap;
+    uint64_t routes, route_cap;
+};
+constexpr size_t kPlanWorkBytes = wide_plan_words(kMaxRows * kTopk) * 4;
+
+// Lays the per-call arrays out behind `base` (which may be null: then only the sizes are wanted).
+Workspace carve(uint8_t* base, const Shape& s) {
+    Workspace w{};
+    size_t at = 0;
+    auto take = [&](size_t bytes) {
+        uint8_t* p = base ? base + at : nullptr;
+        at += (bytes + 255) & ~size_t(255);
+        return p;
+    };
+    w.tiles = tiles_for(s.rows);
+    w.routes = uint64_t(s.rows) * kTopk;
+    w.route_cap = uint64_t(capacity_class(s.rows)) * kTopk;
+    w.group_cap = uint32_t(group_bound(w.routes));
+    w.chunk_cap = uint32_t(chunk_bound(w.routes, w.tiles));
+    const uint64_t I = s.inter, gcap = w.group_cap, ccap = w.chunk_cap;
+    // The tile kernels ask for their chunk record, row table and row verdicts before they know whether the
+    // chunk exists: those tables cover the whole grid (chunk capacity rounded up to runs on eight XCDs).
+    const uint64_t grid_chunks = ccap + 8 * kTileRun;
+    w.plan_work = reinterpret_cast<uint32_t*>(take(kPlanWorkBytes));
+    w.inverse = reinterpret_cast<int32_t*>(take(w.bytes[0] = w.route_cap * 4));
+    w.original = reinterpret_cast<int32_t*>(take(w.bytes[1] = w.route_cap * 4));
+    w.grouped_weights = reinterpret_cast<float*>(take(w.bytes[2] = w.route_cap * 4));
+    w.groups = reinterpret_cast<Group*>(take(w.bytes[3] = gcap * sizeof(Group)));
+    w.chunks = reinterpret_cast<Chunk*>(take(w.bytes[11] = grid_chunks * sizeof(Chunk)));
+    w.dq = take(w.bytes[5] = gcap * 16 * I);
+    w.dqs = take(w.bytes[6] = gcap * 16 * I / 32);
+    w.y = reinterpret_cast<float*>(take(w.bytes[7] = w.routes * kHidden * 4));
+    if (w.tiles > 2 && !s.conforming) {
+        w.xg = take(ccap * gathered_scale_bytes(kHidden));
+        w.dg = take(ccap * gathered_scale_bytes(s.inter));
+        w.rowbad = reinterpret_cast<uint32_t*>(take(grid_chunks * 16 * 4));
+        w.xrows = reinterpret_cast<int32_t*>(take(grid_chunks * 128 * 4));
+        w.yrows = reinterpret_cast<int32_t*>(take(ccap * 128 * 4));
+    }
+    if (s.taps) {
+        w.tap_gate = reinterpret_cast<float*>(take(w.bytes[8] = gcap * 16 * I * 4));
+        w.tap_up = reinterpret_cast<float*>(take(w.bytes[9] = gcap * 16 * I * 4));
+        w.tap_h = reinterpret_cast<float*>(take(w.bytes[10] = gcap * 16 * I * 4));
+    }
+    if (s.host_io) {
+        w.x = take(size_t(s.rows) * kHidden);
+        w.xs = take(size_t(s.rows) * (kHidden / 32));
+        w.ids = reinterpret_cast<int32_t*>(take(w.routes * 4));
+        w.weights = reinterpret_cast<float*>(take(w.routes * 4));
+        w.bf16 = reinterpret_cast<uint16_t*>(take(size_t(s.rows) * kHidden * 2));
+    }
+    w.total = at;
+    return w;
+}
+
 // Kernels whose dynamic LDS passes 64 KB need the limit raised once per process.
 bool lds_ready = false;
-uint32_t compute_units = 0;  // of the device the first scratch was made on
-hipError_t plan_lds_attr() {
+hipError_t raise_lds_limits() {
     if (lds_ready) return hipSuccess;
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(plan_kernel),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, int(kMaxRows * kTopk));
@@ -68,13 +169,6 @@ hipError_t plan_lds_attr() {
     if (e == hipSuccess)
         e = hipFuncSetAttribute(reinterpret_cast<const void*>(fc2_tile_kernel),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, int(kTileLdsBytes));
-    if (e == hipSuccess)
-        e = hipFuncSetAttribute(reinterpret_cast<const void*>(fc2_stream_kernel),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, int(kStreamLdsBytes));
-    int device = 0, cus = 0;
-    if (e == hipSuccess) e = hipGetDevice(&device);
-    if (e == hipSuccess) e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device);
-    compute_units = uint32_t(cus);
     lds_ready = e == hipSuccess;
     return e;
 }
@@ -89,255 +183,245 @@ struct m26s_b1_layer {
 };
 
 struct m26s_b1_scratch {
-    hipStream_t st = nullptr;
+    hipStream_t stream = nullptr;
     bool own_stream = false;
-    hipEvent_t e0 = nullptr, ep = nullptr, ea = nullptr, ec = nullptr, e1 = nullptr;
-    Dev x, xs, iw, inv, orig, gw, groups, chunks, meta, dq, dqs, y, bf16, pad, tap_gate, tap_up, tap_h, xg, rowbad, dg, planw, xrows, yrows, big;
-    std::vector<uint8_t> hiw;
+    hipEvent_t begun = nullptr, planned = nullptr, fc1_done = nullptr, fc2_done = nullptr, ended = nullptr;
+    uint8_t* fixed = nullptr;  // kFixedBytes
+    uint8_t* slab = nullptr;
+    size_t slab_bytes = 0;
+    Workspace last{};  // of the latest call, for the views
     bool taps = false;
-    bool stream_fc2 = false;  // FC2's large chunks through the persistent kernel of b1_stream.h
-    uint32_t last_rows = 0, last_inter = 0;
+    uint32_t last_rows = 0;
 };
 
 namespace {
 
-int layer_build(const Canonical& c, uint32_t inter, m26s_b1_layer** out, char* err, size_t errlen) {
+// The slab only grows. Growing it frees the old one, which waits for the device: calls still in flight on it finish first.
+int fit_slab(m26s_b1_scratch* S, size_t bytes, Outcome& out) {
+    if (bytes <= S->slab_bytes) return 0;
+    if (S->slab) (void)hipFree(S->slab);
+    S->slab = nullptr;
+    S->slab_bytes = 0;
+    M26G_TRY(out, hipMalloc(reinterpret_cast<void**>(&S->slab), bytes), "b1 workspace alloc");
+    S->slab_bytes = bytes;
+    // The wide planner's first word is its fault key, armed to "none"; its scan re-arms it after every call.
+    M26G_TRY(out, hipMemsetAsync(S->slab, 0xff, 16, S->stream), "b1 workspace arm");
+    return 0;
+}
+
+int layer_build(const Canonical& c, uint32_t inter, m26s_b1_layer** made, Outcome& out) {
     auto* L = new (std::nothrow) m26s_b1_layer();
-    if (!L) { set_msg(err, errlen, "b1 layer: host allocation failed"); return 2; }
+    if (!L) return out.fail(2, "b1 layer: host allocation failed");
     L->lay.inter = inter;
-    hipError_t e = hipMalloc(reinterpret_cast<void**>(&L->prepared), L->lay.bytes() * kExperts);
-    if (e != hipSuccess) { set_err(err, errlen, "b1 layer prepared alloc", e); delete L; return 2; }
     uint32_t* flag = nullptr;
-    uint32_t h = 1;
-    std::vector<uint8_t> present(kExperts, 1);
-    if ((e = hipMalloc(reinterpret_cast<void**>(&L->resident), kExperts)) != hipSuccess ||
-        (e = hipMemcpy(L->resident, present.data(), kExperts, hipMemcpyHostToDevice)) != hipSuccess ||
-        (e = hipMalloc(reinterpret_cast<void**>(&flag), 4)) != hipSuccess ||
-        (e = hipMemset(flag, 0, 4)) != hipSuccess) {
-        set_err(err, errlen, "b1 layer metadata", e);
-        m26s_b1_layer_free(L);
-        return 2;
+    uint32_t abnormal = 1;
+    const std::vector<uint8_t> present(kExperts, 1);  // expert id == slot: every expert of the pool is resident
+    hipError_t e = hipMalloc(reinterpret_cast<void**>(&L->prepared), L->lay.bytes() * kExperts);
+    const char* step = "b1 layer prepared alloc";
+    if (e == hipSuccess) { step = "b1 layer metadata"; e = hipMalloc(reinterpret_cast<void**>(&L->resident), kExperts); }
+    if (e == hipSuccess) e = hipMemcpy(L->resident, present.data(), kExperts, hipMemcpyHostToDevice);
+    if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void**>(&flag), 4);
+    if (e == hipSuccess) e = hipMemset(flag, 0, 4);
+    if (e == hipSuccess) {
+        step = "b1 prepare";
+        prepare_kernel<<<dim3(inter / 8, kExperts), 256>>>(c, L->prepared, L->lay, flag);
+        e = hipGetLastError();
     }
-    prepare_kernel<<<dim3(inter / 8, kExperts), 256>>>(c, L->prepared, L->lay, flag);
-    if ((e = hipGetLastError()) != hipSuccess || (e = hipMemcpy(&h, flag, 4, hipMemcpyDeviceToHost)) != hipSuccess ||
-        (e = hipDeviceSynchronize()) != hipSuccess) {
-        (void)hipFree(flag);
-        set_err(err, errlen, "b1 prepare", e);
+    if (e == hipSuccess) e = hipMemcpy(&abnormal, flag, 4, hipMemcpyDeviceToHost);
+    if (e == hipSuccess) e = hipDeviceSynchronize();
+    if (flag) (void)hipFree(flag);
+    if (e != hipSuccess) {
         m26s_b1_layer_free(L);
-        return 2;
+        return out.runtime(e, step);
     }
-    (void)hipFree(flag);
-    L->all_normal = h == 0;
-    *out = L;
+    L->all_normal = abnormal == 0;
+    *made = L;
     return 0;
 }
 
-int scratch_build(hipStream_t stream, bool own, m26s_b1_scratch** out, char* err, size_t errlen) {
-    if (!out) { set_msg(err, errlen, "b1 scratch: null out"); return 1; }
+int scratch_build(hipStream_t stream, bool own, m26s_b1_scratch** made, Outcome& out) {
+    if (!made) return out.fail(1, "b1 scratch: null out");
     auto* S = new (std::nothrow) m26s_b1_scratch();
-    if (!S) { set_msg(err, errlen, "b1 scratch: host allocation failed"); return 1; }
-    hipError_t e = hipSuccess;
-    S->st = stream;
+    if (!S) return out.fail(1, "b1 scratch: host allocation failed");
+    S->stream = stream;
     S->own_stream = own;
-    if ((own && (e = hipStreamCreateWithFlags(&S->st, hipStreamNonBlocking)) != hipSuccess) ||
-        (e = hipEventCreate(&S->e0)) != hipSuccess || (e = hipEventCreate(&S->ep)) != hipSuccess ||
-        (e = hipEventCreate(&S->ea)) != hipSuccess || (e = hipEventCreate(&S->ec)) != hipSuccess ||
-        (e = hipEventCreate(&S->e1)) != hipSuccess || (e = S->meta.ensure(kMetaWords * 4)) != hipSuccess ||
-        (e = S->pad.ensure(8192 + 256)) != hipSuccess ||
-        (e = hipMemset(S->pad.p, 0, 8192)) != hipSuccess ||
-        (e = hipMemset(S->pad.as<uint8_t>() + 8192, 127, 256)) != hipSuccess || (e = plan_lds_attr()) != hipSuccess) {
-        set_err(err, errlen, "b1 scratch stream/events", e);
-        m26s_b1_scratch_free(S);
-        return 1;
+    hipError_t e = own ? hipStreamCreateWithFlags(&S->stream, hipStreamNonBlocking) : hipSuccess;
+    for (hipEvent_t* ev : {&S->begun, &S->planned, &S->fc1_done, &S->fc2_done, &S->ended})
+        if (e == hipSuccess) e = hipEventCreate(ev);
+    if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void**>(&S->fixed), kFixedBytes);
+    if (e == hipSuccess) e = raise_lds_limits();
+    if (e == hipSuccess) {
+        fixed_init_kernel<<<1, 256, 0, S->stream>>>(S->fixed);
+        e = hipGetLastError();
     }
-    meta_reset_kernel<<<1, 64, 0, S->st>>>(S->meta.as<uint32_t>());
-    if ((e = hipGetLastError()) != hipSuccess || (e = hipDeviceSynchronize()) != hipSuccess) {
-        set_err(err, errlen, "b1 scratch meta", e);
+    if (e == hipSuccess) e = hipStreamSynchronize(S->stream);
+    if (e != hipSuccess) {
         m26s_b1_scratch_free(S);
-        return 1;
+        return out.fail(1, "b1 scratch stream/events: %s", hipGetErrorString(e));
     }
-    *out = S;
+    *made = S;
     return 0;
 }
 
-#define M26S_CK(expr, what) do { if ((e = (expr)) != hipSuccess) { set_err(err, errlen, what, e); return 2; } } while (0)
+// What one call launches on, whoever owns the memory: the scratch handle's slab or the static workspace.
+struct Launch {
+    hipStream_t stream;
+    Fixed fixed;
+    Workspace ws;
+    bool taps;
+    hipEvent_t planned, fc1_done, fc2_done;  // null: not timed
+};
 
+void mark(hipEvent_t ev, hipStream_t st) { if (ev) (void)hipEventRecord(ev, st); }
+
+PlanView plan_view(const Launch& k) {
+    return PlanView{k.ws.inverse, k.ws.original, k.ws.grouped_weights, k.ws.groups, k.ws.chunks, k.fixed.meta};
+}
+
+Fc1Args fc1_args(const m26s_b1_layer* L, const Launch& k, const uint8_t* x, size_t xp, const uint8_t* xs, size_t xsp) {
+    return Fc1Args{L->prepared, L->lay, plan_view(k), x, xp, xs, xsp, k.fixed.zero_row, k.fixed.unit_scales, k.ws.dq, k.ws.dqs,
+                   k.taps ? k.ws.tap_gate : nullptr, k.taps ? k.ws.tap_up : nullptr, k.taps ? k.ws.tap_h : nullptr,
+                   k.ws.xg, k.ws.rowbad, k.ws.xrows, k.ws.dg};
+}
+Fc2Args fc2_args(const m26s_b1_layer* L, const Launch& k) {
+    return Fc2Args{L->prepared, L->lay, plan_view(k), k.ws.dq, k.ws.dqs, k.fixed.zero_row, k.fixed.unit_scales, k.ws.y,
+                   uint32_t(k.ws.routes), k.ws.dg, k.ws.yrows, k.ws.rowbad};
+}
+
+// Decode-size calls: every wave streams its own weight block from HBM, activations from L2.
 template <int NT>
-void launch_ffn(const m26s_b1_layer* L, m26s_b1_scratch* S, const PlanView& pv, const uint8_t* x, size_t xp,
-                const uint8_t* xs, size_t xsp, uint32_t chunk_cap, uint64_t routes) {
-    const uint8_t* zero = S->pad.as<uint8_t>();
-    Fc1Args f1{L->prepared, L->lay, pv, x, xp, xs, xsp, zero, zero + 8192, S->dq.as<uint8_t>(), S->dqs.as<uint8_t>(),
-               S->taps ? S->tap_gate.as<float>() : nullptr, S->taps ? S->tap_up.as<float>() : nullptr,
-               S->taps ? S->tap_h.as<float>() : nullptr, nullptr, nullptr, nullptr, nullptr};
-    fc1_kernel<NT><<<dim3(L->lay.inter / 128, chunk_cap), 256, 0, S->st>>>(f1);
-    (void)hipEventRecord(S->ea, S->st);
-    Fc2Args f2{L->prepared, L->lay, pv, S->dq.as<uint8_t>(), S->dqs.as<uint8_t>(), zero, zero + 8192,
-               S->y.as<float>(), uint32_t(routes), nullptr, nullptr, nullptr, 0};
-    fc2_kernel<NT><<<dim3(16 / kFc2Blocks, chunk_cap), 256, 0, S->st>>>(f2);
-    (void)hipEventRecord(S->ec, S->st);
+void launch_direct(const m26s_b1_layer* L, const Launch& k, const Fc1Args& f1, const Fc2Args& f2) {
+    fc1_kernel<NT><<<dim3(L->lay.inter / 128, k.ws.chunk_cap), 256, 0, k.stream>>>(f1);
+    mark(k.fc1_done, k.stream);
+    fc2_kernel<NT><<<dim3(16 / kFc2Blocks, k.ws.chunk_cap), 256, 0, k.stream>>>(f2);
+    mark(k.fc2_done, k.stream);
 }
-
 // Prefill-size calls: workgroups that share each chunk's activation tiles through LDS, two per compute unit.
-void launch_tiles(const m26s_b1_layer* L, m26s_b1_scratch* S, const PlanView& pv, const uint8_t* x, size_t xp,
-                  const uint8_t* xs, size_t xsp, uint32_t chunk_cap, uint64_t routes) {
-    const uint8_t* zero = S->pad.as<uint8_t>();
-    const uint32_t inter = L->lay.inter;
-    // Full-intermediate layers hand FC2's large chunks to the persistent stream kernel (b1_stream.h).
-    const bool stream = S->stream_fc2 && inter == kStreamSteps * 128 && compute_units >= 8;
-    gather_scales_kernel<<<chunk_cap, 256, 0, S->st>>>(pv, xs, xsp, S->xg.as<uint32_t>(), S->rowbad.as<uint32_t>(),
-                                                     S->xrows.as<int32_t>(), S->yrows.as<int32_t>(),
-                                                     stream ? S->big.as<int32_t>() : nullptr);
-    Fc1Args f1{L->prepared, L->lay, pv, x, xp, xs, xsp, zero, zero + 8192, S->dq.as<uint8_t>(), S->dqs.as<uint8_t>(),
-               S->taps ? S->tap_gate.as<float>() : nullptr, S->taps ? S->tap_up.as<float>() : nullptr,
-               S->taps ? S->tap_h.as<float>() : nullptr, S->xg.as<uint8_t>(), S->rowbad.as<uint32_t>(), S->xrows.as<int32_t>(),
-               S->dg.as<uint8_t>()};
-    fc1_tile_kernel<<<tile_grid(inter / 128, chunk_cap), kTileThreads, kTileLdsBytes, S->st>>>(f1);
-    (void)hipEventRecord(S->ea, S->st);
-    Fc2Args f2{L->prepared, L->lay, pv, S->dq.as<uint8_t>(), S->dqs.as<uint8_t>(), zero, zero + 8192,
-               S->y.as<float>(), uint32_t(routes), S->dg.as<uint8_t>(), S->yrows.as<int32_t>(), S->rowbad.as<uint32_t>(), 0};
-    if (stream) {
-        fc2_stream_kernel<<<compute_units / 8 * 8, kStreamThreads, kStreamLdsBytes, S->st>>>(StreamArgs{f2, S->big.as<BigChunk>()});
-        f2.skip_from = kStreamFromGroups;
-    }
-    fc2_tile_kernel<<<tile_grid(kHidden / 256, chunk_cap), kTileThreads, kTileLdsBytes, S->st>>>(f2);
-    (void)hipEventRecord(S->ec, S->st);
+void launch_tiles(const m26s_b1_layer* L, const Launch& k, const Fc1Args& f1, const Fc2Args& f2) {
+    gather_scales_kernel<<<k.ws.chunk_cap, 256, 0, k.stream>>>(f1.plan, f1.xs, f1.xs_pitch, reinterpret_cast<uint32_t*>(k.ws.xg),
+                                                              k.ws.rowbad, k.ws.xrows, k.ws.yrows);
+    fc1_tile_kernel<<<tile_grid(L->lay.inter / 128, k.ws.chunk_cap), kTileThreads, kTileLdsBytes, k.stream>>>(f1);
+    mark(k.fc1_done, k.stream);
+    fc2_tile_kernel<<<tile_grid(kHidden / 256, k.ws.chunk_cap), kTileThreads, kTileLdsBytes, k.stream>>>(f2);
+    mark(k.fc2_done, k.stream);
+}
+// Layers with exceptional weight scales: decode-then-multiply, group by group.
+void launch_conforming(const m26s_b1_layer* L, const Launch& k, const Fc1Args& f1, const Fc2Args& f2) {
+    fc1_conform_kernel<<<dim3(L->lay.inter / kConformColumns, k.ws.group_cap), kConformColumns, 0, k.stream>>>(f1);
+    mark(k.fc1_done, k.stream);
+    fc2_conform_kernel<<<dim3(kHidden / kConformColumns, k.ws.group_cap), kConformColumns, 0, k.stream>>>(f2);
+    mark(k.fc2_done, k.stream);
 }
 
-// Enqueue plan -> FC1(+quantizer) -> FC2 -> reduce on device-resident inputs. No host wait.
-int enqueue(const m26s_b1_layer* L, m26s_b1_scratch* S, const uint8_t* x, size_t xp, const uint8_t* xs, size_t xsp,
-            const int32_t* ids, const float* w, uint32_t rows, uint16_t* bf16_out, float* partial, char* err,
-            size_t errlen) {
-    hipError_t e;
-    const uint32_t cap = capacity_class(rows), nt = tiles_for(rows), inter = L->lay.inter;
-    const uint64_t routes = uint64_t(rows) * kTopk, route_cap = uint64_t(cap) * kTopk;
-    const uint64_t gcap = group_bound(routes), ccap = chunk_bound(routes, nt);
-    M26S_CK(S->inv.ensure(route_cap * 4), "b1 inv alloc");
-    M26S_CK(S->orig.ensure(route_cap * 4), "b1 orig alloc");
-    M26S_CK(S->gw.ensure(route_cap * 4), "b1 gw alloc");
-    M26S_CK(S->groups.ensure(route_cap * sizeof(Group)), "b1 groups alloc");
-    M26S_CK(S->chunks.ensure(route_cap * sizeof(Chunk)), "b1 chunks alloc");
-    // Eight groups of slack behind the intermediate and one spare row behind y: the stream kernel reads
-    // all eight tiles of a chunk whatever its group count, and parks the rows that hold no token.
-    M26S_CK(S->dq.ensure((gcap + 8) * 16 * inter), "b1 dq alloc");
-    M26S_CK(S->dqs.ensure(gcap * 16 * inter / 32), "b1 dqs alloc");
-    M26S_CK(S->y.ensure((routes + 1) * kHidden * 4), "b1 y alloc");
-    if (nt > 2) {
-        M26S_CK(S->xg.ensure(ccap * gathered_scale_bytes(kHidden)), "b1 gathered input scales alloc");
-        M26S_CK(S->dg.ensure(ccap * gathered_scale_bytes(inter)), "b1 gathered intermediate scales alloc");
-        // The tile kernels fetch these beside their chunk record, before they know whether the chunk exists:
-        // the tables cover the whole grid (chunk capacity rounded up to runs on eight XCDs).
-        M26S_CK(S->rowbad.ensure((ccap + 8 * kTileRun) * 16 * 4), "b1 row verdict alloc");
-        M26S_CK(S->xrows.ensure((ccap + 8 * kTileRun) * 128 * 4), "b1 chunk row table alloc");
-        M26S_CK(S->yrows.ensure(ccap * 128 * 4), "b1 chunk route table alloc");
-        M26S_CK(S->big.ensure((ccap + 1) * sizeof(BigChunk)), "b1 large chunk list alloc");
-    }
-    if (S->taps) {
-        M26S_CK(S->tap_gate.ensure(gcap * 16 * inter * 4), "b1 gate tap alloc");
-        M26S_CK(S->tap_up.ensure(gcap * 16 * inter * 4), "b1 up tap alloc");
-        M26S_CK(S->tap_h.ensure(gcap * 16 * inter * 4), "b1 h tap alloc");
-    }
-    const PlanView pv{S->inv.as<int32_t>(), S->orig.as<int32_t>(), S->gw.as<float>(), S->groups.as<Group>(),
-                      S->chunks.as<Chunk>(), S->meta.as<uint32_t>()};
-    M26S_CK(hipEventRecord(S->e0, S->st), "b1 event 0");
-    // Stage faults accumulate across enqueued calls until the next sync; only the plan words reset.
+// plan -> FC1 (+ quantizer) -> FC2 -> combine on device-resident inputs. Launches only.
+hipError_t launch_ffn(const m26s_b1_layer* L, const Launch& k, const uint8_t* x, size_t xp, const uint8_t* xs, size_t xsp,
+                      const int32_t* ids, const float* w, uint32_t rows, uint16_t* bf16_out, float* partial) {
+    const PlanView pv = plan_view(k);
+    const uint32_t nt = k.ws.tiles, routes = uint32_t(k.ws.routes);
     if (rows > kWidePlanFrom) {  // several compute units share the scatter (b1_kernels.h, "Stage 1 for large calls")
-        const void* before = S->planw.p;
-        M26S_CK(S->planw.ensure(wide_plan_words(uint32_t(route_cap)) * 4), "b1 plan work alloc");
-        if (S->planw.p != before) M26S_CK(hipMemsetAsync(S->planw.p, 0xff, 16, S->st), "b1 plan work arm");  // a new buffer: no fault yet
-        const uint32_t wide = wide_plan_groups(uint32_t(routes));
-        plan_count_kernel<<<wide, kPlanThreads, 0, S->st>>>(ids, w, rows, L->resident, S->planw.as<uint32_t>());
-        plan_scan_kernel<<<1, kPlanThreads, 0, S->st>>>(uint32_t(routes), S->planw.as<uint32_t>(), pv, nt);
-        plan_place_kernel<<<wide, kPlanThreads, 0, S->st>>>(ids, w, rows, S->planw.as<uint32_t>(), pv, S->taps);
+        const uint32_t wide = wide_plan_groups(routes);
+        plan_count_kernel<<<wide, kPlanThreads, 0, k.stream>>>(ids, w, rows, L->resident, k.ws.plan_work);
+        plan_scan_kernel<<<1, kPlanThreads, 0, k.stream>>>(routes, k.ws.plan_work, pv, nt);
+        plan_place_kernel<<<wide, kPlanThreads, 0, k.stream>>>(ids, w, rows, k.ws.plan_work, pv, k.taps);
     } else {
-        plan_kernel<<<1, kPlanThreads, routes, S->st>>>(ids, w, rows, L->resident, pv, nt, 0, S->taps);
+        plan_kernel<<<1, kPlanThreads, routes, k.stream>>>(ids, w, rows, L->resident, pv, nt, 0, k.taps);
     }
-    M26S_CK(hipGetLastError(), "b1 plan launch");
-    M26S_CK(hipEventRecord(S->ep, S->st), "b1 event p");
-    if (nt == 1) launch_ffn<1>(L, S, pv, x, xp, xs, xsp, uint32_t(ccap), routes);
-    else if (nt == 2) launch_ffn<2>(L, S, pv, x, xp, xs, xsp, uint32_t(ccap), routes);
-    else launch_tiles(L, S, pv, x, xp, xs, xsp, uint32_t(ccap), routes);
-    M26S_CK(hipGetLastError(), "b1 fc launch");
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    mark(k.planned, k.stream);
+    const Fc1Args f1 = fc1_args(L, k, x, xp, xs, xsp);
+    const Fc2Args f2 = fc2_args(L, k);
+    if (!L->all_normal) launch_conforming(L, k, f1, f2);
+    else if (nt == 1) launch_direct<1>(L, k, f1, f2);
+    else if (nt == 2) launch_direct<2>(L, k, f1, f2);
+    else launch_tiles(L, k, f1, f2);
+    if ((e = hipGetLastError()) != hipSuccess) return e;
     const uint64_t n4 = uint64_t(rows) * (kHidden / 4);
     const uint32_t blocks = uint32_t(n4 / 256 < 65536 ? (n4 + 255) / 256 : 65536);
-    reduce_kernel<<<blocks, 256, 0, S->st>>>(S->y.as<float>(), w, rows, partial, bf16_out,
-                                             S->meta.as<uint32_t>() + kReduceFault, S->meta.as<uint32_t>());
-    M26S_CK(hipGetLastError(), "b1 reduce launch");
-    M26S_CK(hipEventRecord(S->e1, S->st), "b1 event 1");
+    reduce_kernel<<<blocks, 256, 0, k.stream>>>(k.ws.y, w, rows, partial, bf16_out, k.fixed.meta + kReduceFault, k.fixed.meta);
+    return hipGetLastError();
+}
+
+// Sizes the scratch for the call, then launches it. Faults of all calls since the last sync accumulate in the meta words.
+int enqueue(const m26s_b1_layer* L, m26s_b1_scratch* S, bool host_io, const uint8_t* x, size_t xp, const uint8_t* xs,
+            size_t xsp, const int32_t* ids, const float* w, uint32_t rows, uint16_t* bf16_out, float* partial, Outcome& out) {
+    const Shape shape{rows, L->lay.inter, S->taps, host_io, !L->all_normal};
+    if (const int rc = fit_slab(S, carve(nullptr, shape).total, out)) return rc;
+    S->last = carve(S->slab, shape);
     S->last_rows = rows;
-    S->last_inter = inter;
+    const Launch k{S->stream, fixed_at(S->fixed), S->last, S->taps, S->planned, S->fc1_done, S->fc2_done};
+    if (host_io) {  // the inputs were staged into the slab by the caller of this function
+        x = S->last.x, xp = kHidden, xs = S->last.xs, xsp = kHidden / 32, ids = S->last.ids, w = S->last.weights;
+        bf16_out = S->last.bf16;
+    }
+    M26G_TRY(out, hipEventRecord(S->begun, S->stream), "b1 event");
+    M26G_TRY(out, launch_ffn(L, k, x, xp, xs, xsp, ids, w, rows, bf16_out, partial), "b1 launch");
+    M26G_TRY(out, hipEventRecord(S->ended, S->stream), "b1 event");
     return 0;
 }
 
-// Wait, read the eight meta words, translate them (b1_serve.cu:365-368, 551-562) and clear them.
-int finish(m26s_b1_scratch* S, uint32_t* meta_out, char* err, size_t errlen) {
-    hipError_t e;
+// Wait, read the meta words, translate them (b1_serve.cu:365-368, 551-562) and clear them.
+int finish(m26s_b1_scratch* S, uint32_t* meta_out, Outcome& out) {
     uint32_t m[kMetaWords];
-    M26S_CK(hipMemcpyAsync(m, S->meta.p, sizeof m, hipMemcpyDeviceToHost, S->st), "b1 meta download");
-    M26S_CK(hipStreamSynchronize(S->st), "b1 compute sync");
-    meta_reset_kernel<<<1, 64, 0, S->st>>>(S->meta.as<uint32_t>());
-    M26S_CK(hipGetLastError(), "b1 meta reset");
+    M26G_TRY(out, hipMemcpyAsync(m, S->fixed, sizeof m, hipMemcpyDeviceToHost, S->stream), "b1 meta download");
+    M26G_TRY(out, hipStreamSynchronize(S->stream), "b1 compute sync");
+    meta_reset_kernel<<<1, 64, 0, S->stream>>>(reinterpret_cast<uint32_t*>(S->fixed));
+    M26G_TRY(out, hipGetLastError(), "b1 meta reset");
     if (meta_out) std::memcpy(meta_out, m, sizeof m);
-    if (m[kPlanFault]) { set_msg(err, errlen, "b1 plan: invalid routes (id/residency/weight/duplicate)"); return 3; }
-    if (S->last_rows && !m[kGroupCount]) { set_msg(err, errlen, "b1 plan: bad group count"); return 3; }
-    if (err && errlen) {
-        if (m[kFc1Fault]) std::snprintf(err, errlen, "b1 fc1 fault %u (groups %u)", m[kFc1Fault], m[kGroupCount]);
-        else if (m[kQuantFault])
-            std::snprintf(err, errlen, "b1 quantizer fault %u at word %u (groups %u)", m[kQuantFault] & 1 ? 1u : 2u,
-                          m[kQuantWhere], m[kGroupCount]);
-        else if (m[kFc2Fault]) std::snprintf(err, errlen, "b1 fc2 fault %u (groups %u)", m[kFc2Fault], m[kGroupCount]);
-        else if (m[kReduceFault]) std::snprintf(err, errlen, "b1 reduce fault %u (groups %u)", m[kReduceFault], m[kGroupCount]);
-    }
-    return (m[kFc1Fault] | m[kQuantFault] | m[kFc2Fault] | m[kReduceFault]) ? 4 : 0;
+    const bool called = S->last_rows != 0;  // a sync with nothing enqueued since the last one has nothing to report
+    S->last_rows = 0;
+    if (m[kPlanFault]) return out.fail(3, "b1 plan: invalid routes (id/residency/weight/duplicate)");
+    if (called && !m[kGroupCount]) return out.fail(3, "b1 plan: bad group count");
+    if (m[kFc1Fault]) return out.fail(4, "b1 fc1 fault %u (groups %u)", m[kFc1Fault], m[kGroupCount]);
+    if (m[kQuantFault])
+        return out.fail(4, "b1 quantizer fault %u at word %u (groups %u)", m[kQuantFault] & 1 ? 1u : 2u, m[kQuantWhere], m[kGroupCount]);
+    if (m[kFc2Fault]) return out.fail(4, "b1 fc2 fault %u (groups %u)", m[kFc2Fault], m[kGroupCount]);
+    if (m[kReduceFault]) return out.fail(4, "b1 reduce fault %u (groups %u)", m[kReduceFault], m[kGroupCount]);
+    return 0;
 }
 
+using Clock = std::chrono::steady_clock;
+float ms_between(Clock::time_point a, Clock::time_point b) { return std::chrono::duration<float, std::milli>(b - a).count(); }
+
+// ms[8]: upload + plan, GPU compute, tail, group count, FC1 (with the fused quantizer), 0, FC2, combine.
 void report(m26s_b1_scratch* S, float* ms, float host_front, float host_total, uint32_t groups) {
     if (!ms) return;
-    float plan = 0, gpu = 0, ph[3] = {0, 0, 0};
-    (void)hipEventElapsedTime(&plan, S->e0, S->ep);
-    (void)hipEventElapsedTime(&gpu, S->ep, S->e1);
-    (void)hipEventElapsedTime(&ph[0], S->ep, S->ea);
-    (void)hipEventElapsedTime(&ph[1], S->ea, S->ec);
-    (void)hipEventElapsedTime(&ph[2], S->ec, S->e1);
-    ms[0] = host_front + plan;
-    ms[1] = gpu;
-    ms[2] = host_total - host_front - plan - gpu;
-    if (ms[2] < 0) ms[2] = 0;
-    ms[3] = float(groups);
-    ms[4] = ph[0];
-    ms[5] = 0.0f;  // the intermediate quantizer runs inside FC1
-    ms[6] = ph[1];
-    ms[7] = ph[2];
+    float plan = 0, gpu = 0, fc1 = 0, fc2 = 0, combine = 0;
+    (void)hipEventElapsedTime(&plan, S->begun, S->planned);
+    (void)hipEventElapsedTime(&gpu, S->planned, S->ended);
+    (void)hipEventElapsedTime(&fc1, S->planned, S->fc1_done);
+    (void)hipEventElapsedTime(&fc2, S->fc1_done, S->fc2_done);
+    (void)hipEventElapsedTime(&combine, S->fc2_done, S->ended);
+    const float tail = host_total - host_front - plan - gpu;
+    const float v[8] = {host_front + plan, gpu, tail < 0 ? 0 : tail, float(groups), fc1, 0.0f, fc2, combine};
+    std::memcpy(ms, v, sizeof v);
 }
 
-bool layer_usable(const m26s_b1_layer* L, char* err, size_t errlen) {
-    if (L->all_normal) return true;
-    set_msg(err, errlen, "b1 ffn: layer holds weight scale bytes outside [2,252]; no conforming path for them yet");
-    return false;
+bool bad_call(const void* L, const void* S, uint32_t rows, size_t pp, size_t sp, const void* a, const void* b, const void* c,
+              const void* d, const void* e) {
+    return !L || !S || !rows || rows > kMaxRows || pp < kHidden || sp < kHidden / 32 || !a || !b || !c || !d || !e;
 }
 
 }  // namespace
 
 extern "C" {
 
-int m26s_b1_layer_new(const uint8_t* canonical_dev, uint64_t canonical_bytes, uint32_t rank, m26s_b1_layer** out,
+int m26s_b1_layer_new(const uint8_t* canonical_dev, uint64_t canonical_bytes, uint32_t rank, m26s_b1_layer** made,
                       char* err, size_t errlen) {
-    if (!canonical_dev || canonical_bytes != uint64_t(kExperts) * kImageBytes || rank >= 4 || !out) {
-        set_msg(err, errlen, "b1 layer: bad canonical extent/rank");
-        return 1;
-    }
-    Canonical c{{canonical_dev, nullptr, nullptr, nullptr}, 1};
-    return layer_build(c, kRankI, out, err, errlen);
+    Outcome out(err, errlen);
+    if (!canonical_dev || canonical_bytes != uint64_t(kExperts) * kImageBytes || rank >= 4 || !made)
+        return out.fail(1, "b1 layer: bad canonical extent/rank");
+    return layer_build(Canonical{{canonical_dev, nullptr, nullptr, nullptr}, 1}, kRankI, made, out);
 }
 
-int m26s_b1_layer_new_full(const uint8_t* const rank_images_dev[4], uint64_t bytes_each, m26s_b1_layer** out,
-                           char* err, size_t errlen) {
-    if (!rank_images_dev || !out || bytes_each != uint64_t(kExperts) * kImageBytes || !rank_images_dev[0] ||
-        !rank_images_dev[1] || !rank_images_dev[2] || !rank_images_dev[3]) {
-        set_msg(err, errlen, "b1 layer: bad canonical extent/rank");
-        return 1;
-    }
-    Canonical c{{rank_images_dev[0], rank_images_dev[1], rank_images_dev[2], rank_images_dev[3]}, 4};
-    return layer_build(c, 4 * kRankI, out, err, errlen);
+int m26s_b1_layer_new_full(const uint8_t* const rank_images_dev[4], uint64_t bytes_each, m26s_b1_layer** made, char* err,
+                           size_t errlen) {
+    Outcome out(err, errlen);
+    if (!rank_images_dev || !made || bytes_each != uint64_t(kExperts) * kImageBytes || !rank_images_dev[0] ||
+        !rank_images_dev[1] || !rank_images_dev[2] || !rank_images_dev[3])
+        return out.fail(1, "b1 layer: bad canonical extent/rank");
+    return layer_build(Canonical{{rank_images_dev[0], rank_images_dev[1], rank_images_dev[2], rank_images_dev[3]}, 4},
+                       4 * kRankI, made, out);
 }
 
 int m26s_b1_layer_all_normal(const m26s_b1_layer* L) { return L && L->all_normal ? 1 : 0; }
@@ -358,87 +442,80 @@ void m26s_b1_layer_free(m26s_b1_layer* L) {
     delete L;
 }
 
-int m26s_b1_scratch_new(m26s_b1_scratch** out, char* err, size_t errlen) {
-    return scratch_build(nullptr, true, out, err, errlen);
+int m26s_b1_scratch_new(m26s_b1_scratch** made, char* err, size_t errlen) {
+    Outcome out(err, errlen);
+    return scratch_build(nullptr, true, made, out);
 }
-int m26s_b1_scratch_new_on(void* hip_stream, m26s_b1_scratch** out, char* err, size_t errlen) {
-    return scratch_build(static_cast<hipStream_t>(hip_stream), false, out, err, errlen);
+int m26s_b1_scratch_new_on(void* hip_stream, m26s_b1_scratch** made, char* err, size_t errlen) {
+    Outcome out(err, errlen);
+    return scratch_build(static_cast<hipStream_t>(hip_stream), false, made, out);
 }
+void* m26s_b1_scratch_stream(const m26s_b1_scratch* S) { return S ? static_cast<void*>(S->stream) : nullptr; }
 
 void m26s_b1_scratch_free(m26s_b1_scratch* S) {
     if (!S) return;
-    for (hipEvent_t ev : {S->e0, S->ep, S->ea, S->ec, S->e1})
+    for (hipEvent_t ev : {S->begun, S->planned, S->fc1_done, S->fc2_done, S->ended})
         if (ev) (void)hipEventDestroy(ev);
-    if (S->own_stream && S->st) (void)hipStreamDestroy(S->st);
+    if (S->slab) (void)hipFree(S->slab);
+    if (S->fixed) (void)hipFree(S->fixed);
+    if (S->own_stream && S->stream) (void)hipStreamDestroy(S->stream);
     delete S;
 }
 
 int m26s_b1_ffn(const m26s_b1_layer* L, m26s_b1_scratch* S, const uint8_t* payload, size_t payload_pitch,
                 const uint8_t* scales, size_t scales_pitch, const int32_t* ids, const float* weights, uint32_t rows,
                 uint16_t* bf16_out, float* ms, char* err, size_t errlen) {
-    if (!L || !S || !rows || rows > kMaxRows || payload_pitch < 4096 || scales_pitch < 128 || !payload || !scales ||
-        !ids || !weights || !bf16_out) {
-        set_msg(err, errlen, "b1 ffn: bad rows/handles/pitch");
-        return 1;
-    }
-    if (!layer_usable(L, err, errlen)) return 4;
-    hipError_t e;
-    const auto t0 = std::chrono::steady_clock::now();
-    const uint64_t routes = uint64_t(rows) * kTopk;
-    M26S_CK(S->x.ensure(size_t(rows) * 4096), "b1 x alloc");
-    M26S_CK(S->xs.ensure(size_t(rows) * 128), "b1 xs alloc");
-    M26S_CK(S->iw.ensure(routes * 8), "b1 ids/w alloc");
-    M26S_CK(S->bf16.ensure(size_t(rows) * 4096 * 2), "b1 bf16 alloc");
-    M26S_CK(hipMemcpy2DAsync(S->x.p, 4096, payload, payload_pitch, 4096, rows, hipMemcpyHostToDevice, S->st), "b1 x upload");
-    M26S_CK(hipMemcpy2DAsync(S->xs.p, 128, scales, scales_pitch, 128, rows, hipMemcpyHostToDevice, S->st), "b1 xs upload");
-    S->hiw.resize(routes * 8);  // ids then weights: one upload (b1_serve.cu:344-347)
-    std::memcpy(S->hiw.data(), ids, routes * 4);
-    std::memcpy(S->hiw.data() + routes * 4, weights, routes * 4);
-    M26S_CK(hipMemcpyAsync(S->iw.p, S->hiw.data(), routes * 8, hipMemcpyHostToDevice, S->st), "b1 ids/w upload");
-    const auto t1 = std::chrono::steady_clock::now();
-    int rc = enqueue(L, S, S->x.as<uint8_t>(), 4096, S->xs.as<uint8_t>(), 128, S->iw.as<int32_t>(),
-                     reinterpret_cast<const float*>(S->iw.as<uint8_t>() + routes * 4), rows, S->bf16.as<uint16_t>(),
-                     nullptr, err, errlen);
-    if (rc) return rc;
-    M26S_CK(hipMemcpyAsync(bf16_out, S->bf16.p, size_t(rows) * 4096 * 2, hipMemcpyDeviceToHost, S->st), "b1 bf16 download");
+    Outcome out(err, errlen);
+    if (bad_call(L, S, rows, payload_pitch, scales_pitch, payload, scales, ids, weights, bf16_out))
+        return out.fail(1, "b1 ffn: bad rows/handles/pitch");
+    const auto t0 = Clock::now();
+    // Stage the caller's host arrays into the slab: rows packed to 4096 / 128 bytes, ids and weights as they are.
+    const Shape shape{rows, L->lay.inter, S->taps, true, !L->all_normal};
+    if (const int rc = fit_slab(S, carve(nullptr, shape).total, out)) return rc;
+    const Workspace ws = carve(S->slab, shape);
+    const size_t routes = size_t(rows) * kTopk;
+    M26G_TRY(out, hipMemcpy2DAsync(ws.x, kHidden, payload, payload_pitch, kHidden, rows, hipMemcpyHostToDevice, S->stream), "b1 x upload");
+    M26G_TRY(out, hipMemcpy2DAsync(ws.xs, kHidden / 32, scales, scales_pitch, kHidden / 32, rows, hipMemcpyHostToDevice, S->stream), "b1 xs upload");
+    M26G_TRY(out, hipMemcpyAsync(ws.ids, ids, routes * 4, hipMemcpyHostToDevice, S->stream), "b1 ids upload");
+    M26G_TRY(out, hipMemcpyAsync(ws.weights, weights, routes * 4, hipMemcpyHostToDevice, S->stream), "b1 weights upload");
+    const auto t1 = Clock::now();
+    if (const int rc = enqueue(L, S, true, nullptr, 0, nullptr, 0, nullptr, nullptr, rows, nullptr, nullptr, out)) return rc;
+    M26G_TRY(out, hipMemcpyAsync(bf16_out, S->last.bf16, size_t(rows) * kHidden * 2, hipMemcpyDeviceToHost, S->stream), "b1 bf16 download");
     uint32_t m[kMetaWords] = {};
-    rc = finish(S, m, err, errlen);
-    const auto t2 = std::chrono::steady_clock::now();
-    report(S, ms, std::chrono::duration<float, std::milli>(t1 - t0).count(),
-           std::chrono::duration<float, std::milli>(t2 - t0).count(), m[kGroupCount]);
+    const int rc = finish(S, m, out);
+    report(S, ms, ms_between(t0, t1), ms_between(t0, Clock::now()), m[kGroupCount]);
     return rc;
 }
 
 int m26s_b1_ffn_enqueue(const m26s_b1_layer* L, m26s_b1_scratch* S, const uint8_t* payload_dev, size_t payload_pitch,
                         const uint8_t* scales_dev, size_t scales_pitch, const int32_t* ids_dev, const float* weights_dev,
                         uint32_t rows, uint16_t* bf16_out_dev, float* partial_dev, char* err, size_t errlen) {
-    if (!L || !S || !rows || rows > kMaxRows || payload_pitch < 4096 || scales_pitch < 128 || !payload_dev ||
-        !scales_dev || !ids_dev || !weights_dev || !bf16_out_dev || (reinterpret_cast<uintptr_t>(payload_dev) & 15) ||
-        (payload_pitch & 15) || (reinterpret_cast<uintptr_t>(scales_dev) & 3) || (scales_pitch & 3)) {
-        set_msg(err, errlen, "b1 ffn: bad rows/handles/pitch");
-        return 1;
-    }
-    if (!layer_usable(L, err, errlen)) return 4;
-    return enqueue(L, S, payload_dev, payload_pitch, scales_dev, scales_pitch, ids_dev, weights_dev, rows, bf16_out_dev,
-                   partial_dev, err, errlen);
+    Outcome out(err, errlen);
+    if (bad_call(L, S, rows, payload_pitch, scales_pitch, payload_dev, scales_dev, ids_dev, weights_dev, bf16_out_dev) ||
+        (reinterpret_cast<uintptr_t>(payload_dev) & 15) || (payload_pitch & 15) ||
+        (reinterpret_cast<uintptr_t>(scales_dev) & 3) || (scales_pitch & 3))
+        return out.fail(1, "b1 ffn: bad rows/handles/pitch");
+    return enqueue(L, S, false, payload_dev, payload_pitch, scales_dev, scales_pitch, ids_dev, weights_dev, rows, bf16_out_dev,
+                   partial_dev, out);
 }
 
 int m26s_b1_scratch_sync(m26s_b1_scratch* S, char* err, size_t errlen) {
-    if (!S) { set_msg(err, errlen, "b1 sync: bad handle"); return 1; }
-    return finish(S, nullptr, err, errlen);
+    Outcome out(err, errlen);
+    if (!S) return out.fail(1, "b1 sync: bad handle");
+    return finish(S, nullptr, out);
 }
 
 int m26s_b1_ffn_dev(const m26s_b1_layer* L, m26s_b1_scratch* S, const uint8_t* payload_dev, size_t payload_pitch,
                     const uint8_t* scales_dev, size_t scales_pitch, const int32_t* ids_dev, const float* weights_dev,
                     uint32_t rows, uint16_t* bf16_out_dev, float* partial_dev, float* ms, char* err, size_t errlen) {
-    const auto t0 = std::chrono::steady_clock::now();
+    const auto t0 = Clock::now();
     int rc = m26s_b1_ffn_enqueue(L, S, payload_dev, payload_pitch, scales_dev, scales_pitch, ids_dev, weights_dev, rows,
                                  bf16_out_dev, partial_dev, err, errlen);
     if (rc) return rc;
+    Outcome out(err, errlen);
     uint32_t m[kMetaWords] = {};
-    rc = finish(S, m, err, errlen);
-    const auto t2 = std::chrono::steady_clock::now();
-    report(S, ms, 0.0f, std::chrono::duration<float, std::milli>(t2 - t0).count(), m[kGroupCount]);
+    rc = finish(S, m, out);
+    report(S, ms, 0.0f, ms_between(t0, Clock::now()), m[kGroupCount]);
     return rc;
 }
 
@@ -446,73 +523,70 @@ int m26s_b1_plan_dev(const int32_t* ids_dev, const float* weights_dev, uint32_t 
                      const uint8_t* resident_dev, int32_t* inverse_dev, int32_t* original_routes_dev,
                      float* grouped_weights_dev, void* groups_dev, uint32_t* group_count_dev, uint32_t* fault_dev,
                      char* err, size_t errlen) {
+    Outcome out(err, errlen);
     if ((capacity != 256 && capacity != 2048 && capacity != 4096 && capacity != 8192) || rows > capacity ||
         !resident_dev || !inverse_dev || !original_routes_dev || !grouped_weights_dev || !groups_dev ||
-        !group_count_dev || !fault_dev || (rows && (!ids_dev || !weights_dev))) {
-        set_msg(err, errlen, "b1 plan: bad capacity/rows/pointers");
-        return 1;
+        !group_count_dev || !fault_dev || (rows && (!ids_dev || !weights_dev)))
+        return out.fail(1, "b1 plan: bad capacity/rows/pointers");
+    // One allocation: the meta words, then the chunk table the planner also fills.
+    uint8_t* work = nullptr;
+    M26G_TRY(out, raise_lds_limits(), "b1 plan lds");
+    M26G_TRY(out, hipMalloc(reinterpret_cast<void**>(&work), 256 + uint64_t(capacity) * kTopk * sizeof(Chunk)), "b1 plan work alloc");
+    uint32_t m[kMetaWords] = {};
+    hipError_t e = hipMemset(work, 0, 256);
+    if (e == hipSuccess) {
+        const PlanView pv{inverse_dev, original_routes_dev, grouped_weights_dev, static_cast<Group*>(groups_dev),
+                          reinterpret_cast<Chunk*>(work + 256), reinterpret_cast<uint32_t*>(work)};
+        plan_kernel<<<1, kPlanThreads, uint64_t(rows) * kTopk, 0>>>(ids_dev, weights_dev, rows, resident_dev, pv, 1,
+                                                                     capacity * kTopk, true);
+        e = hipGetLastError();
     }
-    hipError_t e;
-    Dev meta, chunks;
-    M26S_CK(plan_lds_attr(), "b1 plan lds");
-    M26S_CK(meta.ensure(kMetaWords * 4), "b1 plan meta alloc");
-    M26S_CK(chunks.ensure(uint64_t(capacity) * kTopk * sizeof(Chunk)), "b1 plan chunks alloc");
-    M26S_CK(hipMemset(meta.p, 0, kMetaWords * 4), "b1 plan meta clear");
-    const PlanView pv{inverse_dev, original_routes_dev, grouped_weights_dev, static_cast<Group*>(groups_dev),
-                      chunks.as<Chunk>(), meta.as<uint32_t>()};
-    uint32_t m[kMetaWords];
-    plan_kernel<<<1, kPlanThreads, uint64_t(rows) * kTopk, 0>>>(ids_dev, weights_dev, rows, resident_dev, pv, 1,
-                                                                 capacity * kTopk, true);
-    M26S_CK(hipGetLastError(), "b1 plan launch");
-    M26S_CK(hipMemcpy(m, meta.p, sizeof m, hipMemcpyDeviceToHost), "b1 plan meta download");
-    M26S_CK(hipMemcpy(fault_dev, &m[kPlanFault], 4, hipMemcpyHostToDevice), "b1 plan fault store");
-    if (m[kPlanFault]) return 0;  // a rejected plan changes nothing but the fault word
-    M26S_CK(hipMemcpy(group_count_dev, &m[kGroupCount], 4, hipMemcpyHostToDevice), "b1 plan count store");
-    return 0;
+    if (e == hipSuccess) e = hipMemcpy(m, work, sizeof m, hipMemcpyDeviceToHost);
+    if (e == hipSuccess) e = hipMemcpy(fault_dev, &m[kPlanFault], 4, hipMemcpyHostToDevice);
+    // A rejected plan changes nothing but the fault word.
+    if (e == hipSuccess && !m[kPlanFault]) e = hipMemcpy(group_count_dev, &m[kGroupCount], 4, hipMemcpyHostToDevice);
+    (void)hipFree(work);
+    return out.runtime(e, "b1 plan");
 }
 
 int m26s_b1_quantize_dev(const float* h_dev, uint64_t elements, uint8_t* payload_dev, uint8_t* scales_dev,
                          uint32_t* faults_dev, char* err, size_t errlen) {
-    if (elements % 32 || (elements && (!h_dev || !payload_dev || !scales_dev || !faults_dev))) {
-        set_msg(err, errlen, "b1 quantize: bad extent/pointers");
-        return 1;
-    }
+    Outcome out(err, errlen);
+    if (elements % 32 || (elements && (!h_dev || !payload_dev || !scales_dev || !faults_dev)))
+        return out.fail(1, "b1 quantize: bad extent/pointers");
     if (!elements) return 0;
-    hipError_t e;
     const uint64_t blocks = elements / 32, need = (blocks + 7) / 8;
     quantize_kernel<<<uint32_t(need < 65535 ? need : 65535), 256>>>(h_dev, blocks, payload_dev, scales_dev, faults_dev);
-    M26S_CK(hipGetLastError(), "b1 quantize launch");
-    M26S_CK(hipDeviceSynchronize(), "b1 quantize sync");
+    M26G_TRY(out, hipGetLastError(), "b1 quantize launch");
+    M26G_TRY(out, hipDeviceSynchronize(), "b1 quantize sync");
     return 0;
 }
 
 int m26s_b1_reduce_dev(const float* y_dev, const float* weights_dev, uint32_t rows, float* partial_dev,
                        uint16_t* bf16_dev, uint32_t* fault_dev, char* err, size_t errlen) {
-    if (rows > kMaxRows || !fault_dev || (rows && (!y_dev || !weights_dev || !bf16_dev))) {
-        set_msg(err, errlen, "b1 reduce: bad rows/pointers");
-        return 1;
-    }
-    hipError_t e;
-    M26S_CK(hipMemset(fault_dev, 0, 4), "b1 reduce fault clear");
+    Outcome out(err, errlen);
+    if (rows > kMaxRows || !fault_dev || (rows && (!y_dev || !weights_dev || !bf16_dev)))
+        return out.fail(1, "b1 reduce: bad rows/pointers");
+    M26G_TRY(out, hipMemset(fault_dev, 0, 4), "b1 reduce fault clear");
     if (!rows) return 0;
     const uint64_t n4 = uint64_t(rows) * (kHidden / 4);
     reduce_kernel<<<uint32_t(n4 / 256 < 65536 ? (n4 + 255) / 256 : 65536), 256>>>(y_dev, weights_dev, rows, partial_dev,
                                                                                 bf16_dev, fault_dev, nullptr);
-    M26S_CK(hipGetLastError(), "b1 reduce launch");
-    M26S_CK(hipDeviceSynchronize(), "b1 reduce sync");
+    M26G_TRY(out, hipGetLastError(), "b1 reduce launch");
+    M26G_TRY(out, hipDeviceSynchronize(), "b1 reduce sync");
     return 0;
 }
 
-void m26s_b1_scratch_set_stream(m26s_b1_scratch* S, int on) { if (S) S->stream_fc2 = on != 0; }
 void m26s_b1_scratch_set_taps(m26s_b1_scratch* S, int on) { if (S) S->taps = on != 0; }
 
 int m26s_b1_scratch_view(const m26s_b1_scratch* S, int which, void** dev_ptr, size_t* bytes) {
-    if (!S || !dev_ptr || !bytes) return 1;
-    const Dev* table[] = {&S->inv, &S->orig, &S->gw, &S->groups, &S->meta, &S->dq, &S->dqs, &S->y,
-                          &S->tap_gate, &S->tap_up, &S->tap_h, &S->chunks};
-    if (which < 0 || which >= int(sizeof table / sizeof table[0]) || !table[which]->p) return 1;
-    *dev_ptr = table[which]->p;
-    *bytes = table[which]->n;
+    if (!S || !dev_ptr || !bytes || !S->slab) return 1;
+    const Workspace& w = S->last;
+    void* const table[] = {w.inverse, w.original, w.grouped_weights, w.groups, S->fixed, w.dq, w.dqs, w.y,
+                           w.tap_gate, w.tap_up, w.tap_h, w.chunks};
+    if (which < 0 || which >= int(sizeof table / sizeof table[0]) || !table[which]) return 1;
+    *dev_ptr = table[which];
+    *bytes = which == 4 ? size_t(kMetaWords) * 4 : w.bytes[which];
     return 0;
 }
 

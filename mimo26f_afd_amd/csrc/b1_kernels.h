@@ -293,10 +293,11 @@ plan_kernel(const int32_t* __restrict__ ids, const float* __restrict__ w, uint32
         const uint32_t ng = (cnt[e] + 15) / 16, left = ng - gpc * j;
         p.chunks[ci] = Chunk{int32_t(gbase[e] + gpc * j), int32_t(left < gpc ? left : gpc), int32_t(e), 0};
     }
+    // The fault word is left alone: a rejected plan of an earlier call on this scratch stays on record,
+    // and keeps the stage kernels of every later call out, until the host has read and cleared it.
     if (tid == 0) {
         p.meta[kGroupCount] = ngroups;
         p.meta[kChunkCount] = nchunks;
-        p.meta[kPlanFault] = 0;
     }
 }
 
@@ -444,10 +445,11 @@ plan_scan_kernel(uint32_t routes, uint32_t* __restrict__ work, PlanView p, uint3
         const uint32_t ng = (cnt[ex] + 15) / 16, left = ng - gpc * j;
         p.chunks[ci] = Chunk{int32_t(gbase[ex] + gpc * j), int32_t(left < gpc ? left : gpc), int32_t(ex), 0};
     }
+    // The fault word is left alone: a rejected plan of an earlier call on this scratch stays on record,
+    // and keeps the stage kernels of every later call out, until the host has read and cleared it.
     if (tid == 0) {
         p.meta[kGroupCount] = ngroups;
         p.meta[kChunkCount] = nchunks;
-        p.meta[kPlanFault] = 0;
     }
 }
 
@@ -495,7 +497,7 @@ plan_place_kernel(const int32_t* __restrict__ ids, const float* __restrict__ w, 
     }
 }
 
-// Clears the per-call stage fault words; runs ahead of the planner on the same stream.
+// Clears the count and fault words once the host has read them.
 __global__ void meta_reset_kernel(uint32_t* meta) {
     if (threadIdx.x < kMetaWords) meta[threadIdx.x] = threadIdx.x == kQuantWhere ? 0xffffffffu : 0u;
 }
@@ -679,7 +681,11 @@ __device__ __forceinline__ void gemm_chunk(v4f (&acc)[4][TT], const uint8_t* __r
 // e^t for t <= 0 in binary32: Cody-Waite reduction by ln 2 (two FMAs), the hardware 2^x on the
 // remainder, exponent put back with ldexp. Within 2 ulp of the true value, the accuracy class of the
 // expf the reference's own kernels call (crates/mimo26-expert/kernels/b1/grouped.cu:89).
+// Below -104 the true value is under half the smallest binary32 subnormal, i.e. zero once rounded; the
+// clamp also keeps the reduction's remainder small for arguments as large as a gate can get (2^127),
+// where the multiple of ln 2 would be off by more than the hardware 2^x can take.
 __device__ __forceinline__ float exp_nonpositive(float t) {
+    t = __builtin_fmaxf(t, -104.0f);
     const float n = __builtin_rintf(t * 1.44269504088896340736f);
     float r = __builtin_fmaf(n, -0.693145751953125f, t);
     r = __builtin_fmaf(n, -1.42860682030941723212e-06f, r);
@@ -886,7 +892,6 @@ struct Fc2Args {
     const uint8_t* dg;  // tile schedule only: the intermediate's scales in MFMA lane order (see Fc1Args)
     const int32_t* yrows;  // tile schedule only, [chunk][8 tiles][16]: the route (row of y) of each row, -1 for none
     const uint32_t* rowbad;  // tile schedule only: as in Fc1Args (bit 8+t: tile t holds a token in that row)
-    int32_t skip_from;       // tile schedule only: chunks of at least this many groups belong to the stream kernel (0: none)
 };
 
 // FC2 epilogue of one wave: unweighted FP32 rows back to y[original route].

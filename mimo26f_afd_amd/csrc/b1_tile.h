@@ -36,7 +36,6 @@ namespace m26g {
 constexpr int kTileThreads = 256, kTileWaves = 4, kWeightStages = 2, kActStages = 3;
 constexpr uint32_t kTileLdsBytes = kTileWaves * kWeightStages * 4096 + kActStages * 8 * 2048;
 static_assert(kTileLdsBytes == 80 * 1024, "two workgroups share the 160 KB of a compute unit");
-constexpr int32_t kStreamFromGroups = 5;  // chunks of at least this many groups can go to the stream kernel (b1_stream.h)
 // Bytes of one chunk's gathered activation scales for a K-deep product: [K/512][8][64] dwords.
 __host__ __device__ constexpr uint32_t gathered_scale_bytes(uint32_t k) { return (k / 512) * 2048; }
 
@@ -87,8 +86,7 @@ __device__ __forceinline__ void mfma_acc(v4f& acc, const v4i& a, const v8i& b, u
 // grid (chunk capacity), 256 threads = 8 tiles x 16 rows x 2 halves of a scale row.
 __global__ void __launch_bounds__(256) gather_scales_kernel(PlanView plan, const uint8_t* __restrict__ xs, size_t xs_pitch,
                                                             uint32_t* __restrict__ xg, uint32_t* __restrict__ rowbad,
-                                                            int32_t* __restrict__ xrows, int32_t* __restrict__ yrows,
-                                                            int32_t* __restrict__ big) {
+                                                            int32_t* __restrict__ xrows, int32_t* __restrict__ yrows) {
     __shared__ uint32_t flags[16];
     const uint32_t c = blockIdx.x, tid = threadIdx.x;
     if (plan.meta[kPlanFault] || c >= plan.meta[kChunkCount]) return;
@@ -96,28 +94,6 @@ __global__ void __launch_bounds__(256) gather_scales_kernel(PlanView plan, const
     if (ch.groups < 1 || ch.groups > 8) return;  // FC1 reports the broken chunk
     const uint32_t tt = tid >> 5, r = (tid >> 1) & 15, half = tid & 1;
     if (tid < 16) flags[tid] = 0;
-    // Chunks of five groups and more are also listed for the stream kernel (b1_stream.h), in chunk order,
-    // so neighbours in the list are mostly chunks of one expert: a chunk's place is the number of large
-    // chunks before it (every workgroup counts for itself: the table is a few KB). big[0] holds the
-    // count, records of four words {chunk, expert, first group, groups} follow from big[4].
-    if (big) {
-        __shared__ uint32_t before, total;
-        if (tid == 0) before = total = 0;
-        __syncthreads();
-        uint32_t mine_before = 0, mine_total = 0;
-        for (uint32_t i = tid; i < plan.meta[kChunkCount]; i += 256) {
-            const uint32_t large = plan.chunks[i].groups >= kStreamFromGroups ? 1u : 0u;
-            mine_total += large;
-            mine_before += i < c ? large : 0u;
-        }
-        if (mine_total) atomicAdd(&total, mine_total);
-        if (mine_before) atomicAdd(&before, mine_before);
-        __syncthreads();
-        if (tid == 0) {
-            if (ch.groups >= kStreamFromGroups) *reinterpret_cast<int4*>(big + 4 + 4 * before) = int4{int32_t(c), ch.expert, ch.first_group, ch.groups};
-            if (c == 0) big[0] = int32_t(total);
-        }
-    }
     __syncthreads();
     const int32_t row = int32_t(tt) < ch.groups ? plan.groups[ch.first_group + tt].input_rows[r] : -1;
     if (half == 0) {  // the chunk's rows flattened: FC1 and FC2 find them one load after their chunk index
@@ -505,7 +481,6 @@ __global__ void __launch_bounds__(kTileThreads, 2) fc2_tile_kernel(Fc2Args a) {
         if (lane == 0) atomicOr(&meta[kFc2Fault], 2u);
         return;
     }
-    if (a.skip_from && ch.groups >= a.skip_from) return;  // the stream kernel's share
     if (ch.groups == 1) fc2_body<1>(a, ch, ob, lane);
     else if (ch.groups == 2) fc2_body<2>(a, ch, ob, lane);
     else if (ch.groups <= 4) fc2_tile_body<4>(a, ch, c, ob, wv, lane, lds, verdict);

@@ -61,11 +61,15 @@ int m26c_frame_fill(const int* idx, const float* wts, const uint8_t* payload, co
                     int hid, uint8_t* routes, uint8_t* hidden, int pitch, void* stream) {
     if (t <= 0) return 0;
     if (!idx || !wts || !payload || !scales || !routes || !hidden || topk <= 0 || hid <= 0 || hid % 256 ||
-        pitch < hid + hid / 32 || pitch % 8)
+        pitch < hid + hid / 32 || pitch % 8 || (reinterpret_cast<uintptr_t>(payload) & 15) ||
+        (reinterpret_cast<uintptr_t>(scales) & 7) || (reinterpret_cast<uintptr_t>(hidden) & 7) ||
+        (reinterpret_cast<uintptr_t>(routes) & 3))
         return 1;
-    const long n = long(t) * topk + long(t) * (hid / 8 + hid / 32 / 8);
-    frame_fill_kernel<<<grid_for(n), kThreads, 0, hipStream_t(stream)>>>(idx, wts, payload, scales, t, topk, hid, routes, hidden,
-                                                                        pitch);
+    const int row_groups = (t + 3) / 4;                                   // one wave per hidden row
+    const long route_groups = (long(t) * topk + kThreads - 1) / kThreads;  // one lane per route entry
+    if (row_groups + route_groups > 0x7fffffffL) return 1;
+    frame_fill_kernel<<<unsigned(row_groups + route_groups), kThreads, 0, hipStream_t(stream)>>>(idx, wts, payload, scales, t, topk, hid,
+                                                                                              routes, hidden, pitch, row_groups);
     return launched();
 }
 

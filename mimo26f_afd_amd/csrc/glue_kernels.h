@@ -166,28 +166,39 @@ __global__ void __launch_bounds__(256) encode_hidden_kernel(const float* __restr
 }
 
 // ---- request frame ----------------------------------------------------------------------------------
-// Route entries (row, expert, weight bits; 12 bytes) and hidden rows (payload then scales at `pitch`),
-// eight bytes per store like the reference: the hidden rows start 8- but not always 16-byte aligned.
+// The body of a request frame behind its header and row descriptors: t * topk route entries of twelve
+// bytes (row, expert, weight bits) and t hidden rows (hid payload bytes, then hid / 32 scale bytes) at
+// `pitch`. The first `row_groups` workgroups move hidden rows, one wave per token: payload and scale rows
+// are read in 16-byte pieces, 1 KB per wave and step, and written as two 8-byte halves, because a frame's
+// hidden rows start on 8-byte boundaries only. The remaining workgroups write the route entries, one
+// route per lane; an entry is three dwords at a 4-byte boundary.
 __global__ void __launch_bounds__(256) frame_fill_kernel(const int* __restrict__ idx, const float* __restrict__ wts,
                                                          const uint8_t* __restrict__ payload, const uint8_t* __restrict__ scales,
                                                          int t, int topk, int hid, uint8_t* __restrict__ routes,
-                                                         uint8_t* __restrict__ hidden, int pitch) {
-    const long nr = long(t) * topk;
-    const int row8 = hid / 8, sc8 = hid / 32 / 8;
-    const long nh = long(t) * (row8 + sc8);
-    for (long i = long(blockIdx.x) * blockDim.x + threadIdx.x; i < nr + nh; i += long(gridDim.x) * blockDim.x) {
-        if (i < nr) {
-            uint32_t* e = reinterpret_cast<uint32_t*>(routes + i * 12);
-            e[0] = uint32_t(i / topk);
-            e[1] = uint32_t(idx[i]);
-            e[2] = __float_as_uint(wts[i]);
-        } else {
-            const long j = i - nr, r = j / (row8 + sc8), c = j % (row8 + sc8);
-            const uint2* src = c < row8 ? reinterpret_cast<const uint2*>(payload + r * hid) + c
-                                        : reinterpret_cast<const uint2*>(scales + r * (hid / 32)) + (c - row8);
-            *reinterpret_cast<uint2*>(hidden + r * pitch + c * 8) = *src;
+                                                         uint8_t* __restrict__ hidden, int pitch, int row_groups) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    if (int(blockIdx.x) < row_groups) {
+        const int token = blockIdx.x * 4 + wave;
+        if (token >= t) return;
+        uint8_t* dst = hidden + size_t(token) * pitch;
+        const uint4* src = reinterpret_cast<const uint4*>(payload + size_t(token) * hid);
+        for (int piece = lane; piece < hid / 16; piece += 64) {
+            const uint4 v = src[piece];
+            uint2* out = reinterpret_cast<uint2*>(dst + piece * 16);
+            out[0] = make_uint2(v.x, v.y);
+            out[1] = make_uint2(v.z, v.w);
         }
+        const uint2* ssrc = reinterpret_cast<const uint2*>(scales + size_t(token) * (hid / 32));
+        for (int piece = lane; piece < hid / 256; piece += 64)
+            reinterpret_cast<uint2*>(dst + hid)[piece] = ssrc[piece];
+        return;
     }
+    const long route = long(blockIdx.x - row_groups) * 256 + threadIdx.x;
+    if (route >= long(t) * topk) return;
+    uint32_t* entry = reinterpret_cast<uint32_t*>(routes + route * 12);
+    entry[0] = uint32_t(route / topk);
+    entry[1] = uint32_t(idx[route]);
+    entry[2] = __float_as_uint(wts[route]);
 }
 
 // ---- rank sum, residual, BF16 cast -----------------------------------------------------------------

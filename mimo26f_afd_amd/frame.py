@@ -298,9 +298,10 @@ class DeviceFrameAdapter:
     checksum of a device-resident frame is not computed here: run such lanes with the checksum off
     (MIMO26_WIRE_NOCRC=1, the reference's fast-path setting) or seal after the frame reaches the host."""
 
-    def __init__(self, layer: b1.Layer, scratch: b1.Scratch, max_rows: int = 8192, stream: int | None = None):
-        """`stream` must be the stream the scratch launches on (the one given to b1.Scratch)."""
-        self.layer, self.scratch, self.max_rows, self.stream = layer, scratch, max_rows, stream
+    def __init__(self, layer: b1.Layer, scratch: b1.Scratch, max_rows: int = 8192):
+        """The route gathering and the staging copy launch on the scratch's own stream, ahead of the
+        FFN that reads what they write; no other stream takes part."""
+        self.layer, self.scratch, self.max_rows, self.stream = layer, scratch, max_rows, scratch.stream
         self.ids = b1.DeviceBuffer(max_rows * TOPK * 4)
         self.weights = b1.DeviceBuffer(max_rows * TOPK * 4)
         self.fault = b1.DeviceBuffer(4)

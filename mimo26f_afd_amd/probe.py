@@ -3,7 +3,7 @@ from __future__ import annotations
 
 import ctypes as C
 
-from ._lib import load
+from ._lib import load_probe
 
 
 class ProbeError(RuntimeError):
@@ -12,7 +12,7 @@ class ProbeError(RuntimeError):
 
 def _run(name: str, *args) -> float:
     value, buf = C.c_double(0.0), C.create_string_buffer(256)
-    rc = getattr(load(), name)(*args, C.byref(value), buf, 256)
+    rc = getattr(load_probe(), name)(*args, C.byref(value), buf, 256)
     if rc != 0:
         raise ProbeError(f"{name}: rc {rc}: {buf.value.decode('utf-8', 'replace')}")
     return value.value

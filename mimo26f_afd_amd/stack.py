@@ -159,18 +159,3 @@ class ResidentStack:
         for layer in self.layers:
             layer.close()
         self.layers = []
-
-
-def reference_rows(seed: int, layer: int, payload: np.ndarray, scales: np.ndarray, ids: np.ndarray,
-                   weights: np.ndarray, oracle):
-    """The CPU rule's BF16 rows for a few tokens of one layer, with that layer's touched experts
-    regenerated on the host. `oracle` is the checker module (tests and the bench pass it in)."""
-    touched = np.unique(ids)
-    pools = []
-    for r in range(4):
-        pool = np.full(synth.EXPERTS * synth.IMAGE_BYTES, 0x22, np.uint8)
-        for e in touched:
-            pool[e * synth.IMAGE_BYTES:(e + 1) * synth.IMAGE_BYTES] = synth.expert_image(seed, r, int(e), layer)
-        pools.append(pool)
-    rc, _, bits, _ = oracle.layer_ffn(pools, payload, scales, ids, weights)
-    return rc, bits

@@ -47,3 +47,19 @@ def run_ffn_dev(layer: b1.Layer, scratch: b1.Scratch, wl: synth.Workload, want_p
     bf = out.to_host(np.uint16).reshape(wl.rows, 4096)
     pf = part.to_host(np.float32).reshape(wl.rows, 4096) if part else None
     return stats, bf, pf
+
+
+def stack_reference_rows(seed: int, layer: int, payload: np.ndarray, scales: np.ndarray, ids: np.ndarray,
+                         weights: np.ndarray):
+    """The CPU rule's BF16 rows for a few tokens of one layer of the resident stack, with that layer's
+    touched experts regenerated on the host from the stack's seeded streams."""
+    import b1_oracle as O
+    touched = np.unique(ids)
+    pools = []
+    for r in range(4):
+        pool = np.full(synth.EXPERTS * synth.IMAGE_BYTES, 0x22, np.uint8)
+        for e in touched:
+            pool[e * synth.IMAGE_BYTES:(e + 1) * synth.IMAGE_BYTES] = synth.expert_image(seed, r, int(e), layer)
+        pools.append(pool)
+    rc, _, bits, _ = O.layer_ffn(pools, payload, scales, ids, weights)
+    return rc, bits

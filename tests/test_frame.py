@@ -125,33 +125,55 @@ def test_return_assembled_in_place():
 
 @pytest.mark.gpu
 def test_serve_request_frames_from_host_and_device_memory():
-    from helpers import DeviceLayer, run_ffn_dev
+    """A request frame served from host memory and from device memory, against the CPU checker's BF16 rows
+    (bars of the benchmark contract); the routes the device gathered are read back and compared with the
+    host parse of the same frame, id for id and weight bit for weight bit."""
+    import b1_oracle as O
+    from helpers import DeviceLayer, bf16_to_f32, parity
     from mimo26f_afd_amd import b1
     wl = synth.make(1)
-    layer = DeviceLayer(wl.pools(wl.touched())).layer
+    pools = wl.pools(wl.touched())
+    layer = DeviceLayer(pools).layer
     scratch = b1.Scratch()
-    _, want, _ = run_ffn_dev(layer, scratch, wl)
+    rc, _, ref_bf16, _ = O.layer_ffn(pools, wl.payload, wl.scales, wl.ids, wl.weights)
+    assert rc == 0
+
+    def check_rows(bits):
+        ma, mr = parity(bf16_to_f32(bits), bf16_to_f32(ref_bf16))
+        assert ma <= 1e-2 and mr <= 1e-3, (ma, mr)
+
     request = F.encode_request(wl.payload, wl.scales, wl.ids, wl.weights, request_id=7, layer_id=3, executor_id=1, seq=4)
     view = F.RequestView.parse(request)
+    host_ids, host_w = F.b1_inputs(view)
+    assert np.array_equal(host_ids, wl.ids) and np.array_equal(host_w.view(np.uint32), wl.weights.view(np.uint32))
     send = np.zeros(128 + wl.rows * 8192, np.uint8)
     stats = F.serve_b1_view(view, layer, scratch, send, seq=11)
     assert stats.groups > 0
     h = F.parse_header(send)
     F.verify_crc(send, 11)
     assert (h["kind"], h["row_count"], h["request_id"], h["layer_id"], h["executor_id"], h["seq"]) == (2, wl.rows, 7, 3, 1, 11)
-    assert np.array_equal(send[128:].view(np.uint16).reshape(wl.rows, 4096), want)
+    served = send[128:].view(np.uint16).reshape(wl.rows, 4096).copy()
+    check_rows(served)
 
     # the same request lying in device memory, at both alignments of its hidden rows (16 rows: rows start
     # 128 + 136 * 16 bytes in, a multiple of 16; shifted by 8 they are not and get staged)
     adapter = F.DeviceFrameAdapter(layer, scratch, max_rows=64)
+    assert adapter.stream == scratch.stream
     for shift in (0, 8):
         dev = b1.DeviceBuffer(request.size + 16)
         assert b1.load().m26s_b1_copy_to_device(dev.ptr + shift, request.ctypes.data, request.size) == 0
         out = b1.DeviceBuffer(128 + wl.rows * 8192)
+        assert b1.load().m26s_b1_copy_to_device(adapter.ids.ptr, np.full(wl.rows * 8, -7, np.int32).ctypes.data, wl.rows * 32) == 0
         header = adapter.serve(request[:128], dev.ptr + shift, out.ptr, seq=12)
+        got_ids = adapter.ids.to_host(np.int32, wl.rows * 8).reshape(wl.rows, 8)
+        got_w = adapter.weights.to_host(np.float32, wl.rows * 8).reshape(wl.rows, 8)
+        assert np.array_equal(got_ids, host_ids), shift                    # what the device gathered = the host parse
+        assert np.array_equal(got_w.view(np.uint32), host_w.view(np.uint32)), shift
         back = out.to_host(np.uint8)
         assert np.array_equal(back[:128], header) and F.parse_header(np.concatenate([header, back[128:]]))["seq"] == 12
-        assert np.array_equal(back[128:].view(np.uint16).reshape(wl.rows, 4096), want), shift
+        rows = back[128:].view(np.uint16).reshape(wl.rows, 4096)
+        check_rows(rows)
+        assert np.array_equal(rows, served), shift                         # and the host-memory path's bits
         dev.free()
         out.free()
     # a frame that breaks the route contract is refused with the row named

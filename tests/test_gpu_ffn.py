@@ -242,27 +242,6 @@ def test_prefill_chunk_properties_and_sampled_parity(full_layer):
     assert np.array_equal(bf_p, bf[perm])
 
 
-def test_stream_schedule_gives_the_default_schedule_bits(full_layer):
-    """The persistent FC2 kernel for chunks of five to eight groups (off by default) reproduces the
-    default schedule bit for bit: configs[3] at 8192 tokens, then a ragged 1000 tokens on the same
-    scratch (smaller second call: few large chunks, most of the work left to the tile kernel)."""
-    _, _, layer = full_layer
-    wl = synth.make(3)
-    pick = np.arange(1000) * 7 % wl.rows
-    small = synth.Workload("ragged", 3, wl.seed, 4, len(pick), wl.ids[pick], wl.weights[pick], wl.x[pick],
-                           wl.payload[pick], wl.scales[pick])
-    s = b1.Scratch()
-    base = [run_ffn_dev(layer, s, w) for w in (wl, small)]
-    s.set_stream(True)
-    for w, (stats0, bf0, pf0) in zip((wl, small), base):
-        stats, bf, pf = run_ffn_dev(layer, s, w)
-        assert stats.groups == stats0.groups
-        assert np.array_equal(bf, bf0) and np.array_equal(pf.view(np.uint32), pf0.view(np.uint32))
-    s.set_stream(False)
-    _, bf, _ = run_ffn_dev(layer, s, small, want_partial=False)
-    assert np.array_equal(bf, base[1][1])
-
-
 def test_two_scratches_in_flight_on_one_layer(full_layer):
     """One scratch is one call in flight; two scratches (two streams) may run at once on the same layer.
     Calls of three sizes (decode schedule, tile schedule) are enqueued alternately without a wait in
@@ -385,14 +364,75 @@ def test_wide_planner_faults_and_recovery(full_layer):
     assert st.groups == int(ref.group_count[0]) and np.array_equal(out2, out)
 
 
-def test_abnormal_weight_scales_are_refused():
-    """A weight scale byte outside [2,252] clears all_normal (b1_fc1_m64.cuh:496-512); the MFMA path is
-    then refused loudly instead of computing with a NaN or saturating scale."""
-    wl = synth.make(1)
+def test_rejected_plan_is_remembered_until_the_sync(full_layer):
+    """Faults of every call enqueued since the last sync accumulate: a call whose routes are rejected,
+    followed by good calls on the same scratch, still makes the sync return code 3, and the later calls
+    compute nothing (their outputs keep the bytes they held); after the sync the scratch is clean. Both
+    planners (one workgroup up to 512 rows, several above)."""
+    wl, _, layer = full_layer
+    big = synth.make(3, rows=640)
+    for w_ in (wl, big):
+        s = b1.Scratch()
+        bad_ids = w_.ids.copy()
+        bad_ids[3, 1] = bad_ids[3, 0]
+        bufs = [b1.DeviceBuffer.from_host(a) for a in (w_.payload, w_.scales, w_.ids, w_.weights, bad_ids)]
+        fill = np.full(w_.rows * 4096, 0xABCD, np.uint16)
+        outs = [b1.DeviceBuffer.from_host(fill) for _ in range(3)]
+        args = (bufs[0].ptr, 4096, bufs[1].ptr, 128)
+        b1.ffn_enqueue(layer, s, *args, bufs[4].ptr, bufs[3].ptr, w_.rows, outs[0].ptr)      # rejected
+        b1.ffn_enqueue(layer, s, *args, bufs[2].ptr, bufs[3].ptr, w_.rows, outs[1].ptr)      # good, but behind a fault
+        with pytest.raises(b1.B1Error, match="invalid routes") as e:
+            s.sync()
+        assert e.value.code == 3
+        assert np.array_equal(outs[0].to_host(np.uint16), fill) and np.array_equal(outs[1].to_host(np.uint16), fill)
+        s.sync()                                                                             # nothing pending: clean
+        b1.ffn_enqueue(layer, s, *args, bufs[2].ptr, bufs[3].ptr, w_.rows, outs[2].ptr)
+        s.sync()
+        _, want, _ = run_ffn_dev(layer, b1.Scratch(), w_, want_partial=False)
+        assert np.array_equal(outs[2].to_host(np.uint16).reshape(w_.rows, 4096), want)
+
+
+def test_four_rank_composition_is_the_reference_sum():
+    """The reference's system: four TP4 ranks each return the BF16 rounding of their own partial row, and
+    the coordinator adds the four planes in rank order in FP32 (crates/mimo26-repack/tests/lattice_oracle.py:94-113,
+    crates/mimo26-coordinator/kernels/glue.cu:200-213). One GPU plays the four ranks in turn (four
+    single-pool layers, configs[2] routing and inputs) and then the coordinator: the rank sum is bit for
+    bit the CPU rule's sum of the GPU's own planes, every plane and the sum meet the bars against the CPU
+    rule's planes and their sum, and the fused layer (one FP32 sum over I = 2048, one BF16 rounding) stays
+    within the wire bound of that sum."""
+    from mimo26f_afd_amd import glue
+    wl = synth.make(2)
     pools = wl.pools(wl.touched())
-    pools[0][int(wl.ids[0, 0]) * synth.IMAGE_BYTES + synth.GATE_SCALES + 5] = 255
-    layer = DeviceLayer(pools).layer
-    assert not layer.all_scales_normal()
-    with pytest.raises(b1.B1Error, match="outside") as e:
-        b1.ffn(layer, b1.Scratch(), wl.payload, wl.scales, wl.ids, wl.weights, wl.rows, np.zeros((wl.rows, 4096), np.uint16))
-    assert e.value.code == 4
+    scratch = b1.Scratch()
+    planes, ref_planes, held = [], [], []
+    for r in range(4):
+        one = synth.Workload(f"rank {r}", 2, wl.seed, 1, wl.rows, wl.ids, wl.weights, wl.x, wl.payload, wl.scales)
+        buf = b1.DeviceBuffer.from_host(pools[r])
+        layer = b1.Layer(buf.ptr, buf.nbytes, r)
+        buf.free()
+        assert layer.intermediate == 512
+        bufs = [b1.DeviceBuffer.from_host(a) for a in (one.payload, one.scales, one.ids, one.weights)]
+        out = b1.DeviceBuffer(wl.rows * 4096 * 2)
+        b1.ffn_dev(layer, scratch, bufs[0].ptr, 4096, bufs[1].ptr, 128, bufs[2].ptr, bufs[3].ptr, wl.rows, out.ptr)
+        held.append(out)
+        planes.append(out.to_host(np.uint16).reshape(wl.rows, 4096))
+        rc, _, ref_bf16, _ = O.layer_ffn([pools[r]], wl.payload, wl.scales, wl.ids, wl.weights)
+        assert rc == 0
+        ref_planes.append(ref_bf16)
+        ma, mr = parity(bf16_to_f32(planes[r]), bf16_to_f32(ref_bf16))
+        assert ma <= MAX_ABS and mr <= MEAN_REL, (r, ma, mr)
+        layer.close()
+    total = b1.DeviceBuffer(wl.rows * 4096 * 4)
+    glue.rank_sum_bf16(*[h.ptr for h in held], total.ptr, wl.rows * 4096, scratch.stream)
+    scratch.sync()
+    got = total.to_host(np.float32).reshape(wl.rows, 4096)
+    assert np.array_equal(got.view(np.uint32), O.rank_sum_bf16(*planes).reshape(wl.rows, 4096).view(np.uint32))
+    want = O.rank_sum_bf16(*ref_planes).reshape(wl.rows, 4096)
+    ma, mr = parity(got, want)
+    assert ma <= MAX_ABS and mr <= MEAN_REL, (ma, mr)
+    # the fused layer against the four-plane sum: each plane carries one BF16 rounding (2^-9 relative)
+    full = DeviceLayer(pools).layer
+    _, _, pf = run_ffn_dev(full, scratch, wl)
+    bound = 2.4e-6 + np.sum([np.abs(bf16_to_f32(p).astype(np.float64)) for p in planes], axis=0) * 2.0 ** -8
+    bound += 1e-4 * np.max(np.abs(want))                                     # FP32 accumulation order (K = 2048 at once against four sums of 512)
+    assert np.all(np.abs(pf.astype(np.float64) - got) <= bound)

@@ -88,16 +88,19 @@ def test_frame_fill_bytes():
     w = rng.random((t, topk)).astype(np.float32)
     payload = rng.integers(0, 256, (t, hid), dtype=np.uint8)
     scales = rng.integers(0, 256, (t, hid // 32), dtype=np.uint8)
-    routes, hidden = D(t * topk * 12), D(t * pitch)
     src = [dev(a) for a in (idx, w, payload, scales)]            # kept alive across the launch
-    glue.frame_fill(*[b.ptr for b in src], t, topk, hid, routes.ptr, hidden.ptr, pitch)
     want = np.zeros((t * topk, 3), np.uint32)
     want[:, 0] = np.repeat(np.arange(t), topk)
     want[:, 1] = idx.reshape(-1)
     want[:, 2] = w.reshape(-1).view(np.uint32)
-    assert np.array_equal(routes.to_host(np.uint32).reshape(-1, 3), want)
-    got = hidden.to_host(np.uint8).reshape(t, pitch)
-    assert np.array_equal(got[:, :hid], payload) and np.array_equal(got[:, hid:hid + hid // 32], scales)
+    for shift in (0, 8):                                         # a frame's hidden rows start on 8-byte boundaries only
+        routes, hidden = D(t * topk * 12 + 16), D(t * pitch + 16)
+        glue.frame_fill(*[b.ptr for b in src], t, topk, hid, routes.ptr + shift // 2, hidden.ptr + shift, pitch)
+        assert np.array_equal(routes.to_host(np.uint8)[shift // 2:shift // 2 + t * topk * 12].view(np.uint32).reshape(-1, 3), want)
+        got = hidden.to_host(np.uint8)[shift:shift + t * pitch].reshape(t, pitch)
+        assert np.array_equal(got[:, :hid], payload) and np.array_equal(got[:, hid:hid + hid // 32], scales)
+    with pytest.raises(glue.GlueError):                          # rows that would start off an 8-byte boundary are refused
+        glue.frame_fill(*[b.ptr for b in src], t, topk, hid, routes.ptr, hidden.ptr + 4, pitch)
 
 
 def test_rank_sum_residual_and_cast_bit_exact():
@@ -154,12 +157,13 @@ def test_chain_router_quantizer_frame_ffn():
 
 def test_roofline_probes_report_plausible_rates():
     """The two measurement aids: a streaming read lands between a third of the HBM peak and the peak,
-    the MFMA-only loop between a third of the FP8 peak and the peak; bad arguments are refused."""
+    the MFMA-only loop between a third of the FP8 peak and a little past it (the nominal 5.0 PFLOP/s is quoted
+    at a lower clock than an idle part boosts to: 4.4 to 5.0 have been measured); bad arguments are refused."""
     from mimo26f_afd_amd import probe
     gbs = probe.read_bandwidth_gbps(1 << 30, 3)
     assert 2600 < gbs < 8000, gbs
     tf = probe.mfma_rate_tflops(500, 2)
-    assert 1600 < tf < 5000, tf
+    assert 1600 < tf < 5000 * 1.1, tf
     with pytest.raises(probe.ProbeError):
         probe.read_bandwidth_gbps(12345, 1)
     with pytest.raises(probe.ProbeError):

@@ -51,7 +51,7 @@ def test_device_pool_matches_host_generator():
 
 @pytest.mark.gpu
 def test_short_stack_against_cpu_rule():
-    import b1_oracle as O
+    from helpers import stack_reference_rows
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     layers, seg, segments, dec_rows = 3, 256, 2, 16
@@ -73,7 +73,7 @@ def test_short_stack_against_cpu_rule():
                         frame = buf["frame"][pick].cpu().numpy()
                         ids, w = routes[l][0][pick].cpu().numpy(), routes[l][1][pick].cpu().numpy()
                         got = buf["out"][pick].view(torch.int16).cpu().numpy().view(np.uint16)
-                        rc, ref = S.reference_rows(st.seed, l, frame[:, :4096].copy(), frame[:, 4096:].copy(), ids, w, O)
+                        rc, ref = stack_reference_rows(st.seed, l, frame[:, :4096].copy(), frame[:, 4096:].copy(), ids, w)
                         assert rc == 0, (kind, l)
                         g = (got.astype(np.uint32) << 16).view(np.float32).astype(np.float64)
                         r = (ref.astype(np.uint32) << 16).view(np.float32).astype(np.float64)
