@@ -105,6 +105,24 @@ int m26s_b1_ffn_enqueue(const m26s_b1_layer* layer, m26s_b1_scratch* scratch, co
 /* Waits for the scratch's stream and decodes the fault words (return codes as above). */
 int m26s_b1_scratch_sync(m26s_b1_scratch* scratch, char* err, size_t errlen);
 
+/* No counterpart in the reference. For callers that cannot allocate: code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc. m26s_b1_ffn_enqueue without a scratch handle: every
+ * per-call array (plan, intermediate, per-route rows, count and fault words) lies in a fixed array of 32 MiB
+ * inside the library's device image, which each GPU the library runs on holds until the process ends, and
+ * the call makes no allocation of any kind. Limits: rows in 1..128 (the decode / verify batch); more rows
+ * return 1 with a message. Launches on `hip_stream` (hipStream_t as void*, NULL = the default stream) and
+ * returns without waiting: 0, 1 for bad arguments, 2 for a runtime error. status_dev (8 uint32 of device
+ * memory, or NULL) receives the call's words {group count, plan fault, chunk count, fc1 fault, quantizer
+ * fault, lowest faulting block, fc2 fault, reduce fault} behind its last kernel: read them after the
+ * stream has run; bf16_out_dev is valid when words 1, 3, 4, 6 and 7 are zero (decoded as m26s_b1_ffn's
+ * return codes 3 and 4). All calls on one GPU share the one array, which keeps the last call's contents
+ * (each call clears the words it needs at zero itself): calls that overlap in time on one GPU race, also
+ * from different streams or threads. Pointers, pitches and alignments as m26s_b1_ffn_enqueue. */
+int m26s_b1_ffn_static(const m26s_b1_layer* layer, const uint8_t* payload_dev, size_t payload_pitch,
+                       const uint8_t* scales_dev, size_t scales_pitch, const int32_t* ids_dev,
+                       const float* weights_dev, uint32_t rows, uint16_t* bf16_out_dev, uint32_t* status_dev,
+                       void* hip_stream, char* err, size_t errlen);
+
 /* ---- stage-level entry points (parity tests and diagnostics) ------------------------------- */
 
 /* Stage 1 alone, on DEVICE arrays: the reference planner's outputs

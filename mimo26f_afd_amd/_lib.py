@@ -35,6 +35,7 @@ SIGNATURES = {
     "m26s_b1_ffn_dev": (C.c_int, [_vp, _vp, _vp, _sz, _vp, _sz, _vp, _vp, C.c_uint32, _vp, _vp, _vp, _cp, _sz]),
     "m26s_b1_ffn_enqueue": (C.c_int, [_vp, _vp, _vp, _sz, _vp, _sz, _vp, _vp, C.c_uint32, _vp, _vp, _cp, _sz]),
     "m26s_b1_scratch_sync": (C.c_int, [_vp, _cp, _sz]),
+    "m26s_b1_ffn_static": (C.c_int, [_vp, _vp, _sz, _vp, _sz, _vp, _vp, C.c_uint32, _vp, _vp, _vp, _cp, _sz]),
     "m26s_b1_plan_dev": (C.c_int, [_vp, _vp, C.c_uint32, C.c_uint32, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _cp, _sz]),
     "m26s_b1_quantize_dev": (C.c_int, [_vp, C.c_uint64, _vp, _vp, _vp, _cp, _sz]),
     "m26s_b1_reduce_dev": (C.c_int, [_vp, _vp, C.c_uint32, _vp, _vp, _vp, _cp, _sz]),

@@ -193,6 +193,19 @@ def ffn_enqueue(layer: Layer, scratch: Scratch, payload_dev: int, payload_pitch:
                                       ids_dev, weights_dev, rows, bf16_out_dev, partial_dev, buf, ERRLEN), buf)
 
 
+STATIC_MAX_ROWS = 128
+
+
+def ffn_static(layer: Layer, payload_dev: int, payload_pitch: int, scales_dev: int, scales_pitch: int, ids_dev: int,
+               weights_dev: int, rows: int, bf16_out_dev: int, status_dev: int | None = None, stream: int | None = None) -> None:
+    """Device-resident call of up to 128 rows that allocates nothing (the workspace is a fixed array inside
+    the library); launches only. `status_dev`: 8 uint32 of device memory that receive the call's count and
+    fault words. Calls that overlap on one GPU race."""
+    buf = _err()
+    _raise(load().m26s_b1_ffn_static(layer._h, payload_dev, payload_pitch, scales_dev, scales_pitch, ids_dev, weights_dev,
+                                     rows, bf16_out_dev, status_dev, stream, buf, ERRLEN), buf)
+
+
 # ---- stage-level entry points -----------------------------------------------------------------
 def plan_dev(ids_dev, weights_dev, rows, capacity, resident_dev, inverse_dev, original_dev, gw_dev, groups_dev,
              count_dev, fault_dev) -> None:

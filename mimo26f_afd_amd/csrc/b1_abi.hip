@@ -404,6 +404,22 @@ bool bad_call(const void* L, const void* S, uint32_t rows, size_t pp, size_t sp,
 
 }  // namespace
 
+// ---- a call that allocates nothing -----------------------------------------------------------------------
+// The workspace of m26s_b1_ffn_static: a fixed array in the library's own device image, so that the call
+// needs no allocation at all. Each GPU the library runs on holds its own copy at its own address from the
+// moment the code object is loaded there until the process ends.
+constexpr uint32_t kStaticRows = 128;            // the decode / verify batch of the benchmark configurations
+constexpr size_t kStaticBytes = size_t(32) << 20;
+static __device__ __align__(256) uint8_t scratch[kStaticBytes];
+
+namespace {
+constexpr int kStaticDevices = 64;
+uint8_t* static_base[kStaticDevices];  // the array's device address per GPU (the symbol itself is no address on the host)
+__global__ void status_copy_kernel(uint32_t* __restrict__ out, const uint32_t* __restrict__ meta) {
+    if (threadIdx.x < kMetaWords) out[threadIdx.x] = meta[threadIdx.x];
+}
+}  // namespace
+
 extern "C" {
 
 int m26s_b1_layer_new(const uint8_t* canonical_dev, uint64_t canonical_bytes, uint32_t rank, m26s_b1_layer** made,
@@ -574,6 +590,45 @@ int m26s_b1_reduce_dev(const float* y_dev, const float* weights_dev, uint32_t ro
                                                                                 bf16_dev, fault_dev, nullptr);
     M26G_TRY(out, hipGetLastError(), "b1 reduce launch");
     M26G_TRY(out, hipDeviceSynchronize(), "b1 reduce sync");
+    return 0;
+}
+
+int m26s_b1_ffn_static(const m26s_b1_layer* L, const uint8_t* payload_dev, size_t payload_pitch, const uint8_t* scales_dev,
+                       size_t scales_pitch, const int32_t* ids_dev, const float* weights_dev, uint32_t rows,
+                       uint16_t* bf16_out_dev, uint32_t* status_dev, void* hip_stream, char* err, size_t errlen) {
+    Outcome out(err, errlen);
+    if (bad_call(L, L, rows, payload_pitch, scales_pitch, payload_dev, scales_dev, ids_dev, weights_dev, bf16_out_dev) ||
+        (reinterpret_cast<uintptr_t>(payload_dev) & 15) || (payload_pitch & 15) ||
+        (reinterpret_cast<uintptr_t>(scales_dev) & 3) || (scales_pitch & 3))
+        return out.fail(1, "b1 ffn: bad rows/handles/pitch");
+    if (rows > kStaticRows)
+        return out.fail(1, "b1 ffn static: %u rows exceed the %u rows the fixed workspace holds", rows, kStaticRows);
+    const Shape shape{rows, L->lay.inter, false, false, !L->all_normal};
+    if (carve(nullptr, shape).total + kFixedBytes > kStaticBytes)
+        return out.fail(1, "b1 ffn static: the call needs more than the fixed workspace of %zu bytes", kStaticBytes);
+    const hipStream_t stream = static_cast<hipStream_t>(hip_stream);
+    int device = -1;
+    M26G_TRY(out, hipGetDevice(&device), "b1 ffn static device");
+    if (device < 0 || device >= kStaticDevices) return out.fail(1, "b1 ffn static: device %d is beyond the %d this entry keeps track of", device, kStaticDevices);
+    if (!static_base[device]) {  // first call on this GPU: find this GPU's copy of the array and write its constants
+        uint8_t* base = nullptr;
+        M26G_TRY(out, hipGetSymbolAddress(reinterpret_cast<void**>(&base), HIP_SYMBOL(scratch)), "b1 ffn static workspace address");
+        if (!base) return out.fail(2, "b1 ffn static workspace address: null");
+        fixed_init_kernel<<<1, 256, 0, stream>>>(base);
+        M26G_TRY(out, hipGetLastError(), "b1 ffn static workspace init");
+        static_base[device] = base;
+    }
+    uint8_t* const base = static_base[device];
+    const Launch k{stream, fixed_at(base), carve(base + kFixedBytes, shape), false, nullptr, nullptr, nullptr};
+    // The array keeps what the last call left: the count and fault words start every call from zero.
+    meta_reset_kernel<<<1, 64, 0, stream>>>(k.fixed.meta);
+    M26G_TRY(out, hipGetLastError(), "b1 ffn static reset");
+    M26G_TRY(out, launch_ffn(L, k, payload_dev, payload_pitch, scales_dev, scales_pitch, ids_dev, weights_dev, rows, bf16_out_dev, nullptr),
+             "b1 ffn static launch");
+    if (status_dev) {
+        status_copy_kernel<<<1, 64, 0, stream>>>(status_dev, k.fixed.meta);
+        M26G_TRY(out, hipGetLastError(), "b1 ffn static status");
+    }
     return 0;
 }
 
