@@ -678,32 +678,33 @@ __device__ __forceinline__ void gemm_chunk(v4f (&acc)[4][TT], const uint8_t* __r
     gemm_blocks<TT>(acc, wp, sp, ksteps, 1, xrow, xsrow, lane, bad, [](int) {});
 }
 
-// e^t for t <= 0 in binary32: Cody-Waite reduction by ln 2 (two FMAs), the hardware 2^x on the
-// remainder, exponent put back with ldexp. Within 2 ulp of the true value, the accuracy class of the
-// expf the reference's own kernels call (crates/mimo26-expert/kernels/b1/grouped.cu:89).
-// Below -104 the true value is under half the smallest binary32 subnormal, i.e. zero once rounded; the
-// clamp also keeps the reduction's remainder small for arguments as large as a gate can get (2^127),
-// where the multiple of ln 2 would be off by more than the hardware 2^x can take.
+// e^t for t <= 0 in binary32 on the hardware 2^x: the product t * log2(e) is formed as a rounded head and
+// its exact remainder (one FMA gives the head's rounding error, a second adds the part of log2(e) that
+// binary32 cannot hold), the head goes through v_exp_f32 and the remainder is applied as a first-order
+// factor. Within 2 ulp of the true value over the whole range, the accuracy class of the expf the
+// reference's own kernels call (crates/mimo26-expert/kernels/b1/grouped.cu:89), in six instructions.
+// Below -104 the true value is under half the smallest binary32 subnormal, i.e. zero once rounded: the
+// clamp keeps the hardware function inside its range for gates as large as 2^127 (an earlier form, a
+// Cody-Waite reduction by ln 2, lost its footing beyond about 2^24 and returned NaN there).
 __device__ __forceinline__ float exp_nonpositive(float t) {
-    t = __builtin_fmaxf(t, -104.0f);
-    const float n = __builtin_rintf(t * 1.44269504088896340736f);
-    float r = __builtin_fmaf(n, -0.693145751953125f, t);
-    r = __builtin_fmaf(n, -1.42860682030941723212e-06f, r);
-    return __builtin_ldexpf(__builtin_amdgcn_exp2f(r * 1.44269504088896340736f), int(n));
+    constexpr float kLog2eHi = 1.44269502162933349609375f, kLog2eLo = 1.925963033500011e-08f, kLn2 = 0.693147182464599609375f;
+    asm("v_max_f32 %0, 0xc2d00000, %0" : "+v"(t));  // max(t, -104) without the NaN canonicalisation fmaxf brings along
+    const float head = t * kLog2eHi;
+    float tail = __builtin_fmaf(t, kLog2eHi, -head);
+    tail = __builtin_fmaf(t, kLog2eLo, tail);
+    const float e = __builtin_amdgcn_exp2f(head);
+    return __builtin_fmaf(e, tail * kLn2, e);
 }
 
 // SwiGLU in the reference's stable form (kernels/b1/grouped.cu:89-93): e = exp(-|g|);
-// s = g >= 0 ? g/(1+e) : (g*e)/(1+e); h = s*u. The quotient is a reciprocal plus one Newton step on
-// the residual (within 1 ulp). The whole activation stays within a few binary32 ulp of the CPU rule,
-// which rounds every step once; the epilogues are bound by vector-instruction issue, and the exactly
-// rounded form costs three times the instructions.
+// s = g >= 0 ? g/(1+e) : (g*e)/(1+e); h = s*u. The quotient is the numerator times the hardware reciprocal
+// (1 ulp). The whole activation stays within a few binary32 ulp of the CPU rule, which rounds every step
+// once; the epilogues are bound by vector-instruction issue, and the exactly rounded form costs three
+// times the instructions.
 __device__ __forceinline__ float silu_up(float g, float u) {
     const float e = exp_nonpositive(g >= 0.0f ? -g : g);
     const float d = 1.0f + e, num = g >= 0.0f ? g : g * e;
-    const float rc = __builtin_amdgcn_rcpf(d);
-    float q = num * rc;
-    q = __builtin_fmaf(__builtin_fmaf(-d, q, num), rc, q);
-    return q * u;
+    return (num * __builtin_amdgcn_rcpf(d)) * u;
 }
 
 struct Fc1Args {
