@@ -11,13 +11,16 @@ and this module checks them on the assembly hipcc emits (no GPU needed):
 
 "In flight" follows the hardware's counters. Vector-memory operations (loads, stores, direct-to-LDS
 loads, whoever issued them) complete in issue order, and `s_waitcnt vmcnt(N)` returns when at most N
-are outstanding: the checker keeps them in a queue and retires all but the newest N at such a wait.
-LDS reads retire at `lgkmcnt(0)`, the only form the kernels use. An MFMA also retires the registers
-it reads: the sources place every MFMA behind the wait for its operands, and the queue model then
-agrees.
+are outstanding: an operation has landed behind such a wait exactly when at least N younger ones were
+issued after it, so the checker keeps, per register in flight, the number of vector-memory operations
+issued since its load. LDS reads retire at `lgkmcnt(0)`, the only form the kernels use. An MFMA also
+retires the registers it reads: the sources place every MFMA behind the wait for its operands.
 
-Each kernel is walked in layout order, twice (loops wrap), which is conservative for the
-straight-line tails. `python -m mimo26f_afd_amd.codegen_check` compiles and checks.
+The walk follows the control flow: the kernel is cut into basic blocks at labels and branches, the state
+at a block's entry is the join over its predecessors (a register is in flight if it is on any path, with
+the smallest count of younger operations any path gives it), iterated to a fixed point, and every
+instruction is then judged against the state that can reach it. `python -m mimo26f_afd_amd.codegen_check`
+compiles and checks.
 """
 from __future__ import annotations
 
@@ -45,6 +48,110 @@ VM_PREFIX = ("global_load", "global_store", "global_atomic", "buffer_", "scratch
 KERNELS = r"^(_ZN4m26g\w*tile_kernel\w*):"
 
 
+BRANCH = re.compile(r"^(s_branch|s_cbranch_\w+)\s+(\.L\w+)")
+CAP = 64  # vmcnt holds six bits: beyond that many younger operations an entry cannot be told apart
+
+
+def _blocks(body: list) -> tuple[list, dict]:
+    """Basic blocks [(label or None, [(line, inasm)])] in layout order and label -> block index."""
+    blocks, cur, label, inasm = [], [], None, False
+    for line in body:
+        text = line.strip()
+        if "ASMSTART" in text:
+            inasm = True
+            continue
+        if "ASMEND" in text:
+            inasm = False
+            continue
+        m = re.match(r"^(\.L\w+):", text)
+        if m:
+            if cur or label is not None:
+                blocks.append((label, cur))
+            cur, label = [], m.group(1)
+            continue
+        if not text or text.startswith(";") or text.startswith("."):
+            continue
+        cur.append((text, inasm))
+        if BRANCH.match(text) or text.startswith("s_endpgm"):
+            blocks.append((label, cur))
+            cur, label = [], None
+    if cur or label is not None:
+        blocks.append((label, cur))
+    return blocks, {lab: i for i, (lab, _) in enumerate(blocks) if lab is not None}
+
+
+def _step(state, text: str, inasm: bool, fn: str, problems):
+    """One instruction on (vm: {reg: younger operations}, lds: set of regs); reports into `problems` if given."""
+    vm, lds = state
+    tok = text.replace(",", " ").split()
+    op = tok[0]
+
+    def issue(regs):
+        for r in list(vm):
+            vm[r] = min(CAP, vm[r] + 1)
+        for r in regs:
+            vm[r] = 0
+
+    if op == "s_waitcnt":
+        m = re.search(r"vmcnt\((\d+)\)", text)
+        if m:
+            n = int(m.group(1))
+            for r in [r for r, y in vm.items() if y >= n]:
+                del vm[r]
+        if "lgkmcnt(0)" in text:
+            lds.clear()
+        return
+    flying = set(vm) | lds
+    if inasm:
+        if op.startswith("ds_read"):
+            lds.update(_regs(tok[1]))
+            return "load"
+        if op.startswith("global_load_dword") and not op.startswith("global_load_lds"):
+            issue(_regs(tok[1]))
+            return "load"
+        if op.startswith(VM_PREFIX):
+            issue(())
+        elif op.startswith("v_mfma"):
+            used = set()
+            for t in tok[2:]:
+                used |= _regs(t)
+            lds.difference_update(used)
+            for r in used:
+                vm.pop(r, None)
+        elif op.startswith(("ds_write", "v_accvgpr")):
+            srcs = set()
+            for t in tok[1:]:
+                srcs |= _regs(t)
+            if problems is not None and srcs & flying:
+                problems.append(f"{fn}: hand-written instruction reads a register with a load in flight: {text}")
+        return
+    if op.startswith(VM_PREFIX):
+        issue(())  # the compiler's own: it waits for them itself, but they hold a place in the order
+    nodest = op.startswith(NO_DEST)
+    dest = set() if nodest or len(tok) < 2 else _regs(tok[1])
+    srcs = set()
+    for t in tok[(1 if nodest else 2):]:
+        srcs |= _regs(t)
+    if problems is not None:
+        if srcs & flying:
+            problems.append(f"{fn}: reads a register with a hand-issued load in flight: {text}")
+        if dest & flying:
+            problems.append(f"{fn}: writes a register with a hand-issued load in flight: {text}")
+
+
+def _join(into, other) -> bool:
+    """Joins `other` into `into`; True if `into` changed."""
+    changed = False
+    for r, y in other[0].items():
+        if r not in into[0] or y < into[0][r]:
+            into[0][r] = y
+            changed = True
+    if not other[1] <= into[1]:
+        into[1].update(other[1])
+        changed = True
+    return changed
+
+
 def check(asm_text: str) -> tuple[dict, list]:
     """Returns ({kernel: hand-issued loads seen}, [problem lines])."""
     funcs, name = {}, None
@@ -60,61 +167,45 @@ def check(asm_text: str) -> tuple[dict, list]:
             funcs[name].append(line)
     seen, problems = {}, []
     for fn, body in funcs.items():
-        vm_queue, flying_lds, inasm, loads = [], set(), False, 0
-        for line in body + body:
-            if "ASMSTART" in line:
-                inasm = True
-                continue
-            if "ASMEND" in line:
-                inasm = False
-                continue
-            tok = line.strip().replace(",", " ").split()
-            if not tok or tok[0].startswith(";") or tok[0].startswith("."):
-                continue
-            op = tok[0]
-            if op == "s_waitcnt":
-                m = re.search(r"vmcnt\((\d+)\)", line)
-                if m:
-                    del vm_queue[:max(0, len(vm_queue) - int(m.group(1)))]
-                if "lgkmcnt(0)" in line:
-                    flying_lds.clear()
-                continue
-            flying = flying_lds.union(*vm_queue) if vm_queue else set(flying_lds)
-            if inasm:
-                if op.startswith("ds_read"):
-                    flying_lds |= _regs(tok[1])
+        blocks, index = _blocks(body)
+        succ = []
+        for i, (_, ins) in enumerate(blocks):
+            last = ins[-1][0] if ins else ""
+            m = BRANCH.match(last)
+            nxt = []
+            if m:
+                if m.group(2) in index:
+                    nxt.append(index[m.group(2)])
+                if m.group(1) != "s_branch" and i + 1 < len(blocks):
+                    nxt.append(i + 1)
+            elif not last.startswith("s_endpgm") and i + 1 < len(blocks):
+                nxt.append(i + 1)
+            succ.append(nxt)
+        entry = [None] * len(blocks)
+        if blocks:
+            entry[0] = ({}, set())
+        work = [0] if blocks else []
+        while work:
+            i = work.pop()
+            state = (dict(entry[i][0]), set(entry[i][1]))
+            for text, inasm in blocks[i][1]:
+                _step(state, text, inasm, fn, None)
+            for j in succ[i]:
+                if entry[j] is None:
+                    entry[j] = (dict(state[0]), set(state[1]))
+                    work.append(j)
+                elif _join(entry[j], state):
+                    work.append(j)
+        loads, found = 0, []
+        for i, (_, ins) in enumerate(blocks):
+            if entry[i] is None:
+                continue  # unreachable
+            state = (dict(entry[i][0]), set(entry[i][1]))
+            for text, inasm in ins:
+                if _step(state, text, inasm, fn, found) == "load":
                     loads += 1
-                elif op.startswith("global_load_dword") and not op.startswith("global_load_lds"):
-                    vm_queue.append(_regs(tok[1]))
-                    loads += 1
-                elif op.startswith(VM_PREFIX):
-                    vm_queue.append(set())
-                elif op.startswith("v_mfma"):
-                    used = set()
-                    for t in tok[2:]:
-                        used |= _regs(t)
-                    flying_lds -= used
-                    for entry in vm_queue:
-                        entry -= used
-                elif op.startswith(("ds_write", "v_accvgpr")):
-                    srcs = set()
-                    for t in tok[1:]:
-                        srcs |= _regs(t)
-                    if srcs & flying:
-                        problems.append(f"{fn}: hand-written instruction reads a register with a load in flight: {line.strip()}")
-                continue
-            if op.startswith(VM_PREFIX):
-                vm_queue.append(set())  # the compiler's own: it waits for them itself, but they hold a place in the order
-            nodest = op.startswith(NO_DEST)
-            dest = set() if nodest or len(tok) < 2 else _regs(tok[1])
-            srcs = set()
-            for t in tok[(1 if nodest else 2):]:
-                srcs |= _regs(t)
-            if srcs & flying:
-                problems.append(f"{fn}: reads a register with a hand-issued load in flight: {line.strip()}")
-            if dest & flying:
-                problems.append(f"{fn}: writes a register with a hand-issued load in flight: {line.strip()}")
-        seen[fn] = loads // 2
+        problems += list(dict.fromkeys(found))
+        seen[fn] = loads
     return seen, problems
 
 

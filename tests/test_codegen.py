@@ -22,7 +22,7 @@ def test_checker_flags_reads_and_writes_under_a_load_in_flight():
     _, p = codegen_check.check(asm(load, wait, mfma, "\tv_mov_b32_e32 v7, v1"))
     assert p == []
     _, p = codegen_check.check(asm(load, "\tv_add_u32_e32 v9, v7, v1", wait, mfma))
-    assert len(p) == 2 and "reads" in p[0]                               # the walk wraps: seen twice
+    assert len(p) == 1 and "reads" in p[0]
     _, p = codegen_check.check(asm(load, "\tv_lshl_add_u64 v[6:7], v[4:5], 0, s[2:3]", wait))
     assert p and "writes" in p[0]                                        # a dead load's register reused
     lds = hand("ds_read_b128 v[20:23], v30 offset:1024")
@@ -50,6 +50,34 @@ def test_checker_retires_vector_memory_operations_in_issue_order():
     assert p == []
     _, p = codegen_check.check(asm(a, lds_load, lds_load, hand("s_waitcnt vmcnt(3)"), "\tv_add_u32_e32 v9, v7, v1", done))
     assert p and "reads" in p[0]
+
+
+def test_checker_follows_the_control_flow():
+    """A register in flight is judged along the paths that can reach an instruction, not along the layout:
+    code that merely follows a branch in the file is not reached from it, a loop's back edge is."""
+    load = hand("global_load_dword v7, v[2:3], off offset:256")
+    wait = hand("s_waitcnt vmcnt(0)")
+    # the load's block jumps over a neighbour in the layout that overwrites v7: not a hazard
+    _, p = codegen_check.check(asm(load, "\ts_branch .LBB0_2", ".LBB0_1:", "\tv_mov_b32_e32 v7, 0", "\ts_endpgm",
+                                   ".LBB0_2:", wait, "\tv_add_u32_e32 v9, v7, v1", "\ts_endpgm"))
+    assert p == []
+    # the same neighbour on the fall-through path of a conditional branch is one
+    _, p = codegen_check.check(asm(load, "\ts_cbranch_scc1 .LBB0_2", ".LBB0_1:", "\tv_mov_b32_e32 v7, 0", "\ts_endpgm",
+                                   ".LBB0_2:", wait, "\ts_endpgm"))
+    assert len(p) == 1 and "writes" in p[0]
+    # a load issued at the bottom of a loop body is still in flight at its top
+    _, p = codegen_check.check(asm(".LBB0_1:", "\tv_add_u32_e32 v9, v7, v1", wait, load, "\ts_cbranch_scc1 .LBB0_1", "\ts_endpgm"))
+    assert len(p) == 1 and "reads" in p[0]
+    _, p = codegen_check.check(asm(".LBB0_1:", wait, "\tv_add_u32_e32 v9, v7, v1", load, "\ts_cbranch_scc1 .LBB0_1", wait, "\ts_endpgm"))
+    assert p == []
+    # two paths join: the register is in flight if it is on either, with the fewer younger operations of the two
+    other = hand("global_load_dword v8, v[2:3], off")
+    _, p = codegen_check.check(asm("\ts_cbranch_scc1 .LBB0_2", load, other, other, "\ts_branch .LBB0_3", ".LBB0_2:", load, other,
+                                   ".LBB0_3:", hand("s_waitcnt vmcnt(2)"), "\tv_add_u32_e32 v9, v7, v1", wait, "\ts_endpgm"))
+    assert len(p) == 1 and "reads" in p[0]                                # on the second path only one operation is younger
+    _, p = codegen_check.check(asm("\ts_cbranch_scc1 .LBB0_2", load, other, other, "\ts_branch .LBB0_3", ".LBB0_2:", load, other,
+                                   ".LBB0_3:", hand("s_waitcnt vmcnt(1)"), "\tv_add_u32_e32 v9, v7, v1", wait, "\ts_endpgm"))
+    assert p == []
 
 
 def test_built_tile_kernels_pass():
