@@ -345,20 +345,23 @@ hipError_t launch_ffn(const m26s_b1_layer* L, const Launch& k, const uint8_t* x,
 }
 
 // Sizes the scratch for the call, then launches it. Faults of all calls since the last sync accumulate in the meta words.
-int enqueue(const m26s_b1_layer* L, m26s_b1_scratch* S, bool host_io, const uint8_t* x, size_t xp, const uint8_t* xs,
+// `timed` brackets the call and its stages with the scratch's events (for the ms[8] report); an untimed call puts
+// nothing but its kernels on the stream: every event is one more packet the GPU's front end works through between two kernels.
+int enqueue(const m26s_b1_layer* L, m26s_b1_scratch* S, bool host_io, bool timed, const uint8_t* x, size_t xp, const uint8_t* xs,
             size_t xsp, const int32_t* ids, const float* w, uint32_t rows, uint16_t* bf16_out, float* partial, Outcome& out) {
     const Shape shape{rows, L->lay.inter, S->taps, host_io, !L->all_normal};
     if (const int rc = fit_slab(S, carve(nullptr, shape).total, out)) return rc;
     S->last = carve(S->slab, shape);
     S->last_rows = rows;
-    const Launch k{S->stream, fixed_at(S->fixed), S->last, S->taps, S->planned, S->fc1_done, S->fc2_done};
+    const Launch k{S->stream, fixed_at(S->fixed), S->last, S->taps, timed ? S->planned : nullptr, timed ? S->fc1_done : nullptr,
+                   timed ? S->fc2_done : nullptr};
     if (host_io) {  // the inputs were staged into the slab by the caller of this function
         x = S->last.x, xp = kHidden, xs = S->last.xs, xsp = kHidden / 32, ids = S->last.ids, w = S->last.weights;
         bf16_out = S->last.bf16;
     }
-    M26G_TRY(out, hipEventRecord(S->begun, S->stream), "b1 event");
+    if (timed) M26G_TRY(out, hipEventRecord(S->begun, S->stream), "b1 event");
     M26G_TRY(out, launch_ffn(L, k, x, xp, xs, xsp, ids, w, rows, bf16_out, partial), "b1 launch");
-    M26G_TRY(out, hipEventRecord(S->ended, S->stream), "b1 event");
+    if (timed) M26G_TRY(out, hipEventRecord(S->ended, S->stream), "b1 event");
     return 0;
 }
 
@@ -543,7 +546,7 @@ int m26s_b1_ffn(const m26s_b1_layer* L, m26s_b1_scratch* S, const uint8_t* paylo
     M26G_TRY(out, hipMemcpyAsync(ws.ids, hids, routes * 4, hipMemcpyHostToDevice, S->stream), "b1 ids upload");
     M26G_TRY(out, hipMemcpyAsync(ws.weights, hweights, routes * 4, hipMemcpyHostToDevice, S->stream), "b1 weights upload");
     const auto t1 = Clock::now();
-    if (const int rc = enqueue(L, S, true, nullptr, 0, nullptr, 0, nullptr, nullptr, rows, nullptr, nullptr, out)) return rc;
+    if (const int rc = enqueue(L, S, true, ms != nullptr, nullptr, 0, nullptr, 0, nullptr, nullptr, rows, nullptr, nullptr, out)) return rc;
     uint16_t* landing = direct ? bf16_out : reinterpret_cast<uint16_t*>(hx + x_bytes + xs_bytes);
     M26G_TRY(out, hipMemcpyAsync(landing, S->last.bf16, out_bytes, hipMemcpyDeviceToHost, S->stream), "b1 bf16 download");
     uint32_t m[kMetaWords] = {};
@@ -553,16 +556,30 @@ int m26s_b1_ffn(const m26s_b1_layer* L, m26s_b1_scratch* S, const uint8_t* paylo
     return rc;
 }
 
-int m26s_b1_ffn_enqueue(const m26s_b1_layer* L, m26s_b1_scratch* S, const uint8_t* payload_dev, size_t payload_pitch,
-                        const uint8_t* scales_dev, size_t scales_pitch, const int32_t* ids_dev, const float* weights_dev,
-                        uint32_t rows, uint16_t* bf16_out_dev, float* partial_dev, char* err, size_t errlen) {
-    Outcome out(err, errlen);
+}  // extern "C"
+
+namespace {
+// The device-pointer call: argument checks, then the launches.
+int enqueue_dev(const m26s_b1_layer* L, m26s_b1_scratch* S, bool timed, const uint8_t* payload_dev, size_t payload_pitch,
+                const uint8_t* scales_dev, size_t scales_pitch, const int32_t* ids_dev, const float* weights_dev, uint32_t rows,
+                uint16_t* bf16_out_dev, float* partial_dev, Outcome& out) {
     if (bad_call(L, S, rows, payload_pitch, scales_pitch, payload_dev, scales_dev, ids_dev, weights_dev, bf16_out_dev) ||
         (reinterpret_cast<uintptr_t>(payload_dev) & 15) || (payload_pitch & 15) ||
         (reinterpret_cast<uintptr_t>(scales_dev) & 3) || (scales_pitch & 3))
         return out.fail(1, "b1 ffn: bad rows/handles/pitch");
-    return enqueue(L, S, false, payload_dev, payload_pitch, scales_dev, scales_pitch, ids_dev, weights_dev, rows, bf16_out_dev,
-                   partial_dev, out);
+    return enqueue(L, S, false, timed, payload_dev, payload_pitch, scales_dev, scales_pitch, ids_dev, weights_dev, rows,
+                   bf16_out_dev, partial_dev, out);
+}
+}  // namespace
+
+extern "C" {
+
+int m26s_b1_ffn_enqueue(const m26s_b1_layer* L, m26s_b1_scratch* S, const uint8_t* payload_dev, size_t payload_pitch,
+                        const uint8_t* scales_dev, size_t scales_pitch, const int32_t* ids_dev, const float* weights_dev,
+                        uint32_t rows, uint16_t* bf16_out_dev, float* partial_dev, char* err, size_t errlen) {
+    Outcome out(err, errlen);
+    return enqueue_dev(L, S, false, payload_dev, payload_pitch, scales_dev, scales_pitch, ids_dev, weights_dev, rows,
+                       bf16_out_dev, partial_dev, out);
 }
 
 int m26s_b1_scratch_sync(m26s_b1_scratch* S, char* err, size_t errlen) {
@@ -575,10 +592,10 @@ int m26s_b1_ffn_dev(const m26s_b1_layer* L, m26s_b1_scratch* S, const uint8_t* p
                     const uint8_t* scales_dev, size_t scales_pitch, const int32_t* ids_dev, const float* weights_dev,
                     uint32_t rows, uint16_t* bf16_out_dev, float* partial_dev, float* ms, char* err, size_t errlen) {
     const auto t0 = Clock::now();
-    int rc = m26s_b1_ffn_enqueue(L, S, payload_dev, payload_pitch, scales_dev, scales_pitch, ids_dev, weights_dev, rows,
-                                 bf16_out_dev, partial_dev, err, errlen);
-    if (rc) return rc;
     Outcome out(err, errlen);
+    int rc = enqueue_dev(L, S, ms != nullptr, payload_dev, payload_pitch, scales_dev, scales_pitch, ids_dev, weights_dev, rows,
+                         bf16_out_dev, partial_dev, out);
+    if (rc) return rc;
     uint32_t m[kMetaWords] = {};
     rc = finish(S, m, out);
     report(S, ms, 0.0f, ms_between(t0, Clock::now()), m[kGroupCount]);
