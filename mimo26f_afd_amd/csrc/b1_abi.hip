@@ -506,16 +506,19 @@ int m26s_b1_ffn(const m26s_b1_layer* L, m26s_b1_scratch* S, const uint8_t* paylo
     const Shape shape{rows, L->lay.inter, S->taps, true, !L->all_normal};
     if (const int rc = fit_slab(S, carve(nullptr, shape).total, out)) return rc;
     const Workspace ws = carve(S->slab, shape);
-    const size_t routes = size_t(rows) * kTopk, x_bytes = size_t(rows) * kHidden, xs_bytes = size_t(rows) * (kHidden / 32),
-                 out_bytes = size_t(rows) * kHidden * 2;
+    const size_t routes = size_t(rows) * kTopk, out_bytes = size_t(rows) * kHidden * 2;
     // The reference's daemon hands over page-locked arrays (its registered receive ring and send slot) and those
     // are copied from and to directly. Pageable arrays go through a page-locked bounce buffer of the scratch:
     // left to the runtime, such copies are staged a piece at a time with a wait after each (2.9 against 0.6 ms
     // for a 128-row call, 158 against 7.7 ms for 8192 rows).
     const bool direct = page_locked(payload) && page_locked(scales) && page_locked(bf16_out);
+    // The staged inputs lie in one run of the slab (rows, scales, ids, weights, each from a 256-byte boundary): the bounce
+    // buffer mirrors that run, so one copy uploads all four.
+    const size_t at_xs = size_t(ws.xs - ws.x), at_ids = size_t(reinterpret_cast<uint8_t*>(ws.ids) - ws.x),
+                 at_w = size_t(reinterpret_cast<uint8_t*>(ws.weights) - ws.x), in_bytes = at_w + routes * 4;
     uint8_t* hx = nullptr;
     if (!direct) {
-        const size_t need = x_bytes + xs_bytes + out_bytes + routes * 8;
+        const size_t need = in_bytes + out_bytes;
         if (need > S->bounce_bytes) {
             if (S->bounce) (void)hipHostFree(S->bounce);
             S->bounce = nullptr;
@@ -526,28 +529,20 @@ int m26s_b1_ffn(const m26s_b1_layer* L, m26s_b1_scratch* S, const uint8_t* paylo
         hx = S->bounce;
         for (uint32_t r = 0; r < rows; ++r) {
             std::memcpy(hx + size_t(r) * kHidden, payload + size_t(r) * payload_pitch, kHidden);
-            std::memcpy(hx + x_bytes + size_t(r) * (kHidden / 32), scales + size_t(r) * scales_pitch, kHidden / 32);
+            std::memcpy(hx + at_xs + size_t(r) * (kHidden / 32), scales + size_t(r) * scales_pitch, kHidden / 32);
         }
-        M26G_TRY(out, hipMemcpyAsync(ws.x, hx, x_bytes, hipMemcpyHostToDevice, S->stream), "b1 x upload");
-        M26G_TRY(out, hipMemcpyAsync(ws.xs, hx + x_bytes, xs_bytes, hipMemcpyHostToDevice, S->stream), "b1 xs upload");
+        std::memcpy(hx + at_ids, ids, routes * 4);
+        std::memcpy(hx + at_w, weights, routes * 4);
+        M26G_TRY(out, hipMemcpyAsync(ws.x, hx, in_bytes, hipMemcpyHostToDevice, S->stream), "b1 input upload");
     } else {
         M26G_TRY(out, hipMemcpy2DAsync(ws.x, kHidden, payload, payload_pitch, kHidden, rows, hipMemcpyHostToDevice, S->stream), "b1 x upload");
         M26G_TRY(out, hipMemcpy2DAsync(ws.xs, kHidden / 32, scales, scales_pitch, kHidden / 32, rows, hipMemcpyHostToDevice, S->stream), "b1 xs upload");
+        M26G_TRY(out, hipMemcpyAsync(ws.ids, ids, routes * 4, hipMemcpyHostToDevice, S->stream), "b1 ids upload");
+        M26G_TRY(out, hipMemcpyAsync(ws.weights, weights, routes * 4, hipMemcpyHostToDevice, S->stream), "b1 weights upload");
     }
-    const void* hids = ids;
-    const void* hweights = weights;
-    if (!direct) {  // the route arrays ride along: ids then weights behind the output's landing area
-        uint8_t* at = hx + x_bytes + xs_bytes + out_bytes;
-        std::memcpy(at, ids, routes * 4);
-        std::memcpy(at + routes * 4, weights, routes * 4);
-        hids = at;
-        hweights = at + routes * 4;
-    }
-    M26G_TRY(out, hipMemcpyAsync(ws.ids, hids, routes * 4, hipMemcpyHostToDevice, S->stream), "b1 ids upload");
-    M26G_TRY(out, hipMemcpyAsync(ws.weights, hweights, routes * 4, hipMemcpyHostToDevice, S->stream), "b1 weights upload");
     const auto t1 = Clock::now();
     if (const int rc = enqueue(L, S, true, ms != nullptr, nullptr, 0, nullptr, 0, nullptr, nullptr, rows, nullptr, nullptr, out)) return rc;
-    uint16_t* landing = direct ? bf16_out : reinterpret_cast<uint16_t*>(hx + x_bytes + xs_bytes);
+    uint16_t* landing = direct ? bf16_out : reinterpret_cast<uint16_t*>(hx + in_bytes);
     M26G_TRY(out, hipMemcpyAsync(landing, S->last.bf16, out_bytes, hipMemcpyDeviceToHost, S->stream), "b1 bf16 download");
     uint32_t m[kMetaWords] = {};
     const int rc = finish(S, m, out);
