@@ -97,7 +97,8 @@ int m26s_b1_ffn_dev(const m26s_b1_layer* layer, m26s_b1_scratch* scratch, const 
 /* Same work, enqueued only: returns after the launches. Faults of every call since the last
  * m26s_b1_scratch_sync accumulate and are reported there: once a call's routes have been rejected or
  * one of its stages has faulted, the later calls enqueued on the scratch before that sync compute
- * nothing, and the sync returns the first fault's code (3 before 4). */
+ * nothing, and the sync returns the first fault's code (3 before 4). The call puts its kernels on the
+ * stream and nothing else (no events: the synchronous entries record theirs only when ms is given). */
 int m26s_b1_ffn_enqueue(const m26s_b1_layer* layer, m26s_b1_scratch* scratch, const uint8_t* payload_dev,
                         size_t payload_pitch, const uint8_t* scales_dev, size_t scales_pitch,
                         const int32_t* ids_dev, const float* weights_dev, uint32_t rows,
