@@ -9,6 +9,15 @@ and this module checks them on the assembly hipcc emits (no GPU needed):
  1. a register with a hand-issued load in flight is not read, and
  2. it is not written: the data in flight would land on top of the new value (an address, say).
 
+ 3. a hand-written MFMA's accumulator is not touched by anything but another MFMA until the matrix pipe
+    has written it back. The MFMAs are `asm` statements too (the accumulator must stay in place), so the
+    compiler does not know that their result arrives eight passes later: a register copy it places
+    right behind the last MFMA of a loop (to hand the accumulator to the code after the loop in another
+    register) reads the value from before that MFMA. The sources put `s_nop` runs where such code can
+    follow; the check counts wait states (one per instruction, N + 1 for `s_nop N`) between a
+    hand-written MFMA and the next non-MFMA access to its destination, and wants at least 12
+    (8 passes + 3, the figure the compiler's own hazard tables hold for this MFMA, and one to spare).
+
 "In flight" follows the hardware's counters. Vector-memory operations (loads, stores, direct-to-LDS
 loads, whoever issued them) complete in issue order, and `s_waitcnt vmcnt(N)` returns when at most N
 are outstanding: an operation has landed behind such a wait exactly when at least N younger ones were
@@ -34,6 +43,17 @@ from . import build
 
 NO_DEST = ("global_load_lds", "global_store", "ds_write", "v_readfirstlane", "v_cmp", "s_", "buffer_store",
            "scratch_store", "global_atomic")
+
+
+MFMA_WAIT_STATES = 12
+
+
+def _aregs(tok: str) -> set:
+    m = re.match(r"a\[(\d+):(\d+)\]", tok)
+    if m:
+        return set(range(int(m.group(1)), int(m.group(2)) + 1))
+    m = re.match(r"a(\d+)$", tok)
+    return {int(m.group(1))} if m else set()
 
 
 def _regs(tok: str) -> set:
@@ -81,10 +101,27 @@ def _blocks(body: list) -> tuple[list, dict]:
 
 
 def _step(state, text: str, inasm: bool, fn: str, problems):
-    """One instruction on (vm: {reg: younger operations}, lds: set of regs); reports into `problems` if given."""
-    vm, lds = state
+    """One instruction on (vm: {reg: younger operations}, lds: set of regs, hot: {accumulator register: wait
+    states since the hand-written MFMA that writes it}); reports into `problems` if given."""
+    vm, lds, hot = state
     tok = text.replace(",", " ").split()
     op = tok[0]
+    mfma = inasm and op.startswith("v_mfma")
+    if hot and not mfma:
+        touched = set()
+        for t in tok[1:]:
+            touched |= _aregs(t)
+        if problems is not None and touched & set(hot):
+            problems.append(f"{fn}: touches an accumulator {min(hot[r] for r in touched & set(hot))} wait states "
+                            f"after the hand-written MFMA that writes it: {text}")
+    states = int(tok[1]) + 1 if op == "s_nop" and len(tok) > 1 and tok[1].isdigit() else 1
+    for r in list(hot):
+        hot[r] += states
+        if hot[r] >= MFMA_WAIT_STATES:
+            del hot[r]
+    if mfma:
+        for r in _aregs(tok[1]):
+            hot[r] = 0
 
     def issue(regs):
         for r in list(vm):
@@ -149,6 +186,10 @@ def _join(into, other) -> bool:
     if not other[1] <= into[1]:
         into[1].update(other[1])
         changed = True
+    for r, y in other[2].items():
+        if r not in into[2] or y < into[2][r]:
+            into[2][r] = y
+            changed = True
     return changed
 
 
@@ -183,16 +224,16 @@ def check(asm_text: str) -> tuple[dict, list]:
             succ.append(nxt)
         entry = [None] * len(blocks)
         if blocks:
-            entry[0] = ({}, set())
+            entry[0] = ({}, set(), {})
         work = [0] if blocks else []
         while work:
             i = work.pop()
-            state = (dict(entry[i][0]), set(entry[i][1]))
+            state = (dict(entry[i][0]), set(entry[i][1]), dict(entry[i][2]))
             for text, inasm in blocks[i][1]:
                 _step(state, text, inasm, fn, None)
             for j in succ[i]:
                 if entry[j] is None:
-                    entry[j] = (dict(state[0]), set(state[1]))
+                    entry[j] = (dict(state[0]), set(state[1]), dict(state[2]))
                     work.append(j)
                 elif _join(entry[j], state):
                     work.append(j)
@@ -200,7 +241,7 @@ def check(asm_text: str) -> tuple[dict, list]:
         for i, (_, ins) in enumerate(blocks):
             if entry[i] is None:
                 continue  # unreachable
-            state = (dict(entry[i][0]), set(entry[i][1]))
+            state = (dict(entry[i][0]), set(entry[i][1]), dict(entry[i][2]))
             for text, inasm in ins:
                 if _step(state, text, inasm, fn, found) == "load":
                     loads += 1

@@ -159,16 +159,21 @@ Workspace carve(uint8_t* base, const Shape& s) {
 
 // Kernels whose dynamic LDS passes 64 KB need the limit raised once per process.
 bool lds_ready = false;
+#ifdef EXP_TILE8
+using TileS = Tile8;
+#else
+using TileS = Tile4;
+#endif
 hipError_t raise_lds_limits() {
     if (lds_ready) return hipSuccess;
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(plan_kernel),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, int(kMaxRows * kTopk));
     if (e == hipSuccess)
-        e = hipFuncSetAttribute(reinterpret_cast<const void*>(fc1_tile_kernel),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, int(kTileLdsBytes));
+        e = hipFuncSetAttribute(reinterpret_cast<const void*>(fc1_tile_kernel<TileS>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, int(TileS::kLdsBytes));
     if (e == hipSuccess)
-        e = hipFuncSetAttribute(reinterpret_cast<const void*>(fc2_tile_kernel),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, int(kTileLdsBytes));
+        e = hipFuncSetAttribute(reinterpret_cast<const void*>(fc2_tile_kernel<TileS>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, int(TileS::kLdsBytes));
     lds_ready = e == hipSuccess;
     return e;
 }
@@ -302,9 +307,9 @@ void launch_direct(const m26s_b1_layer* L, const Launch& k, const Fc1Args& f1, c
 void launch_tiles(const m26s_b1_layer* L, const Launch& k, const Fc1Args& f1, const Fc2Args& f2) {
     gather_scales_kernel<<<k.ws.chunk_cap, 256, 0, k.stream>>>(f1.plan, f1.xs, f1.xs_pitch, reinterpret_cast<uint32_t*>(k.ws.xg),
                                                               k.ws.rowbad, k.ws.xrows, k.ws.yrows);
-    fc1_tile_kernel<<<tile_grid(L->lay.inter / 128, k.ws.chunk_cap), kTileThreads, kTileLdsBytes, k.stream>>>(f1);
+    fc1_tile_kernel<TileS><<<tile_grid(L->lay.inter / (32 * TileS::kWaves), k.ws.chunk_cap), TileS::kThreads, TileS::kLdsBytes, k.stream>>>(f1);
     mark(k.fc1_done, k.stream);
-    fc2_tile_kernel<<<tile_grid(kHidden / 256, k.ws.chunk_cap), kTileThreads, kTileLdsBytes, k.stream>>>(f2);
+    fc2_tile_kernel<TileS><<<tile_grid(kHidden / (64 * TileS::kWaves), k.ws.chunk_cap), TileS::kThreads, TileS::kLdsBytes, k.stream>>>(f2);
     mark(k.fc2_done, k.stream);
 }
 // Layers with exceptional weight scales: decode-then-multiply, group by group.

@@ -33,9 +33,17 @@
 
 namespace m26g {
 
-constexpr int kTileThreads = 256, kTileWaves = 4, kWeightStages = 2, kActStages = 3;
-constexpr uint32_t kTileLdsBytes = kTileWaves * kWeightStages * 4096 + kActStages * 8 * 2048;
-static_assert(kTileLdsBytes == 80 * 1024, "two workgroups share the 160 KB of a compute unit");
+// A tile workgroup's shape: W waves, operands D k-steps ahead. Weight fragments sit in a private ring of D
+// stages per wave (a stage is free once its fragments are in registers), activation fragments in a ring
+// of D + 1 stages shared by the waves (the extra stage decouples the slowest reader from the next load).
+template <int W, int D>
+struct TileShape {
+    static constexpr int kWaves = W, kAhead = D, kThreads = 64 * W, kWeightStages = D, kActStages = D + 1;
+    static constexpr uint32_t kLdsBytes = W * D * 4096 + (D + 1) * 8 * 2048;
+};
+using Tile4 = TileShape<4, 2>;  // 80 KB: two workgroups per compute unit
+using Tile8 = TileShape<8, 3>;  // 160 KB: one workgroup per compute unit, rows shared by eight waves
+static_assert(Tile4::kLdsBytes == 80 * 1024 && Tile8::kLdsBytes == 160 * 1024, "the 160 KB of a compute unit");
 // Bytes of one chunk's gathered activation scales for a K-deep product: [K/512][8][64] dwords.
 __host__ __device__ constexpr uint32_t gathered_scale_bytes(uint32_t k) { return (k / 512) * 2048; }
 
@@ -135,24 +143,30 @@ __global__ void __launch_bounds__(256) gather_scales_kernel(PlanView plan, const
 // per k-step: `row[i]` is this lane's row of tile wv*(TT/4)+i (lane offset 16*(lane/16) included),
 // so the lane that loads a fragment cell is the lane that will hold it. `sx` points at this lane's
 // dword of tile 0, quad 0 of the chunk's gathered activation scales.
-template <int TT>
+template <class S, int TT>
 __device__ __forceinline__ void gemm_chunk_lds(v4f (&acc)[4][TT], const uint8_t* __restrict__ wp,
                                                const uint8_t* __restrict__ sp, const uint8_t* __restrict__ sx, int ksteps,
-                                               const uint8_t* const (&row)[TT / 4], uint32_t wv, uint32_t lane, uint8_t* lds) {
+                                               const uint8_t* const (&row)[(2 * TT / S::kWaves + 1) / 2], uint32_t wv,
+                                               uint32_t lane, uint8_t* lds) {
     static_assert(TT == 4 || TT == 8, "activation tiles per chunk");
-    constexpr int kMine = TT / kTileWaves;  // activation tiles this wave stages
+    constexpr int kWeightStages = S::kWeightStages, kActStages = S::kActStages, kAhead = S::kAhead;
+    // Activation cells (a tile's two 1 KB halves) this wave stages per k-step: cells wv*kCells .. +kCells-1 of the
+    // chunk's 2*TT. With eight waves and four tiles that is half a tile.
+    constexpr int kCells = 2 * TT / S::kWaves;
+    static_assert(kCells >= 1, "every wave stages at least one cell");
     uint8_t* wring = lds + wv * (kWeightStages * 4096);          // [stage][tile][lane][16]
-    uint8_t* aring = lds + kTileWaves * kWeightStages * 4096;    // [stage][tt][half][lane][16]
-    // The direct loads of one k-step: item i < 2*kMine is an activation cell (tile i/2, half i%2),
-    // the other four are the weight rows. A k-step issues exactly kPerStep of them, spread over its
-    // TT groups of MFMAs so the memory pipeline never sees a burst; the waits count on that total.
-    constexpr int kPerStep = 2 * kMine + 4;
+    uint8_t* aring = lds + S::kWaves * kWeightStages * 4096;      // [stage][tt][half][lane][16]
+    // The direct loads of one k-step: item i < kCells is an activation cell, the other four are the weight
+    // rows. A k-step issues exactly kPerStep of them, spread over its TT groups of MFMAs so the memory
+    // pipeline never sees a burst; the waits count on that total.
+    constexpr int kPerStep = kCells + 4;
     auto stage_item = [&](int item, int ks, uint32_t astage, uint32_t wstage) {
-        if (item < 2 * kMine) {
-            const int m = item >> 1, half = item & 1;
-            load_row_to_lds(row[m] + ks * 128 + half * 64, aring + ((astage * TT + wv * kMine + m) * 2 + half) * 1024);
+        if (item < kCells) {
+            const uint32_t cell = wv * kCells + item, half = cell & 1u;  // row[] is indexed from the wave's first tile
+            const int m = int(item + ((wv * kCells) & 1u)) >> 1;
+            load_row_to_lds(row[m] + ks * 128 + half * 64, aring + (astage * TT * 2 + cell) * 1024);
         } else {
-            const int t = item - 2 * kMine;
+            const int t = item - kCells;
             load_row_to_lds(wp + size_t(ks) * 4096 + t * 1024, wring + wstage * 4096 + t * 1024);
         }
     };
@@ -190,9 +204,9 @@ __device__ __forceinline__ void gemm_chunk_lds(v4f (&acc)[4][TT], const uint8_t*
     };
     const int last = ksteps - 1, quads = ksteps / 4;
     load_scales(sw0, sa0, 0);
-    stage_all(0, 0, 0);
-    stage_all(1 < last ? 1 : last, 1, 1);
-    wait_loads_but<kPerStep>();  // step 0 and the first scales have landed, step 1 may still fly
+#pragma unroll
+    for (int d = 0; d < kAhead; ++d) stage_all(d < last ? d : last, d, d);
+    wait_loads_but<(kAhead - 1) * kPerStep>();  // step 0 and the first scales have landed, the later steps may still fly
     read_weights(af[0], 0);
     lds_barrier();
     v4i flo, fhi;  // the fragment a k-step starts with
@@ -201,7 +215,7 @@ __device__ __forceinline__ void gemm_chunk_lds(v4f (&acc)[4][TT], const uint8_t*
     // epilogue instructions otherwise take issue slots from this loop's fragment reads and loads
     // (measured: 2 % off FC1 at 8192 tokens).
     __builtin_amdgcn_s_setprio(3);
-    uint32_t wr = 0, ar = 0;  // weight stage that takes step k+2; activation stage of step k
+    uint32_t wr = 0, ar = 0;  // weight stage of step k, which takes step k+kAhead; activation stage of step k
     int q = 0;
     // One k-step with MFMA scale select b = ks % 4 (an immediate, hence the macro).
     //
@@ -214,11 +228,13 @@ __device__ __forceinline__ void gemm_chunk_lds(v4f (&acc)[4][TT], const uint8_t*
 #define M26G_KSTEP(b, SW, SA)                                                                                  \
     {                                                                                                          \
         const int ks = 4 * q + (b);                                                                            \
-        /* Weights of step k sit in registers, so their stage `wr` takes step k+2; step k+1 is in     */      \
-        /* stage wr^1. Activations: step k reads stage ar, k+1 sits in ar+1, k+2 goes to ar+2.        */      \
-        const uint32_t ar1 = ar == kActStages - 1 ? 0 : ar + 1, ar2 = ar1 == kActStages - 1 ? 0 : ar1 + 1;     \
+        /* Weights of step k sit in registers, so their stage `wr` takes step k+kAhead; step k+1 is   */      \
+        /* in the stage after it. Activations: step k reads stage ar, k+1 sits in the next one, and   */      \
+        /* step k+kAhead goes to the stage before ar, which step k-1 has finished with.               */      \
+        const uint32_t ar1 = ar == kActStages - 1 ? 0 : ar + 1, ar2 = ar == 0 ? kActStages - 1 : ar - 1;       \
+        const uint32_t wr1 = wr == kWeightStages - 1 ? 0 : wr + 1;                                             \
         /* Past the end the last step is staged again into stages nobody reads any more. */                   \
-        const int ahead = ks + 2 < last ? ks + 2 : last;                                                       \
+        const int ahead = ks + kAhead < last ? ks + kAhead : last;                                             \
         const uint32_t fs = aring_at + ar * TT * 2048;                                                         \
         v4i lo = flo, hi = fhi; /* fragment 0, fetched at the end of the step before */                       \
         _Pragma("unroll") for (int tt = 0; tt < TT; ++tt) {                                                    \
@@ -227,12 +243,12 @@ __device__ __forceinline__ void gemm_chunk_lds(v4f (&acc)[4][TT], const uint8_t*
                 _Pragma("unroll") for (int item = 0; item < kPerStep; ++item)                                  \
                     if (item * TT / kPerStep == tt) stage_item(item, ahead, ar2, wr);                          \
                 __builtin_amdgcn_sched_barrier(0);                                                             \
-                /* Everything but this step's own loads (step k+2) has landed: activations and weights */      \
-                /* of step k+1, issued one whole k-step ago, and the next quad's scales, older still.   */      \
-                wait_loads_but<kPerStep>();                                                                    \
+                /* Everything but the loads of the last kAhead-1 steps has landed: activations and     */      \
+                /* weights of step k+1, and the next quad's scales, older still.                        */      \
+                wait_loads_but<(kAhead - 1) * kPerStep>();                                                     \
                 lds_barrier(); /* with the wait for this group's fragment */                                   \
                 read_fragment(flo, fhi, aring_at + ar1 * TT * 2048);                                           \
-                read_weights(af[((b) + 1) & 1], wr ^ 1);                                                       \
+                read_weights(af[((b) + 1) & 1], wr1);                                                          \
             } else {                                                                                           \
                 wait_lds_but<0>();                                                                             \
             }                                                                                                  \
@@ -258,7 +274,7 @@ __device__ __forceinline__ void gemm_chunk_lds(v4f (&acc)[4][TT], const uint8_t*
             lo = nlo;                                                                                          \
             hi = nhi;                                                                                          \
         }                                                                                                      \
-        wr ^= 1;                                                                                               \
+        wr = wr1;                                                                                              \
         ar = ar1;                                                                                              \
     }
     // A quad: fetch the next quad's scales into the other set, then four k-steps on this set.
@@ -270,6 +286,10 @@ __device__ __forceinline__ void gemm_chunk_lds(v4f (&acc)[4][TT], const uint8_t*
         M26G_KSTEP(1, SW, SA)                                                                                  \
         M26G_KSTEP(2, SW, SA)                                                                                  \
         M26G_KSTEP(3, SW, SA)                                                                                  \
+        /* The compiler may put anything behind a quad, a copy of an accumulator included (it hands them to */ \
+        /* the code after the loop in other registers when it likes), and it does not know that the last  */ \
+        /* MFMA's result is eight passes away: twelve wait states cover that.                             */ \
+        asm volatile("s_nop 11" ::: "memory");                                                                \
         ++q;                                                                                                   \
     }
 #pragma unroll 1
@@ -307,10 +327,14 @@ __device__ __forceinline__ uint32_t after_loop(uint32_t lane) {
 // FC1 for chunk c by one workgroup: 128 intermediate columns x 16*TT rows; the wave owns block cb.
 // `token[m]` is the row table's entry for this lane's row of tile wv*(TT/4)+m, fetched by the caller beside
 // the chunk record so that the rows' addresses are one memory latency behind the workgroup's start, not two.
-template <int TT>
+// Activation tiles a wave of shape S stages rows of, per k-step, in a chunk of TT tiles, and the first of them.
+template <class S, int TT> constexpr int staged_tiles() { return (2 * TT / S::kWaves + 1) / 2; }
+template <class S, int TT> __device__ __forceinline__ uint32_t first_staged_tile(uint32_t wv) { return (wv * (2 * TT / S::kWaves)) >> 1; }
+
+template <class S, int TT>
 __device__ __forceinline__ void fc1_tile_body(const Fc1Args& a, const Chunk ch, uint32_t c, uint32_t cb, uint32_t wv,
-                                              uint32_t lane, uint8_t* lds, const int32_t (&token)[TT / kTileWaves]) {
-    constexpr int kMine = TT / kTileWaves;
+                                              uint32_t lane, uint8_t* lds, const int32_t (&token)[staged_tiles<S, TT>()]) {
+    constexpr int kMine = staged_tiles<S, TT>();
     const uint32_t g = lane >> 4;
     const int32_t expert = ch.expert;
     const uint8_t* row[kMine];
@@ -325,7 +349,7 @@ __device__ __forceinline__ void fc1_tile_body(const Fc1Args& a, const Chunk ch, 
     for (int t = 0; t < 4; ++t)
 #pragma unroll
         for (int tt = 0; tt < TT; ++tt) acc[t][tt] = v4f{0.f, 0.f, 0.f, 0.f};
-    gemm_chunk_lds<TT>(acc, wp, sp, sx, int(kHidden / 128), row, wv, lane, lds);
+    gemm_chunk_lds<S, TT>(acc, wp, sp, sx, int(kHidden / 128), row, wv, lane, lds);
     const uint32_t lane2 = after_loop(lane), r2 = lane2 & 15;
     const uint32_t verdict = a.rowbad[c * 16 + r2], bad = verdict & 1u;
     // The accumulators leave the accumulation registers through LDS, sixteen tiles at a time: whole-tile
@@ -334,7 +358,7 @@ __device__ __forceinline__ void fc1_tile_body(const Fc1Args& a, const Chunk ch, 
     // becomes one rolled loop over the activation tiles. Unrolled it is 70 KB of code, and two workgroups
     // in different phases then evict each other's instructions from the cache the compute units share.
     // Every wave has drained its own direct loads; after the barrier nobody's are left, and each wave
-    // takes a quarter of the first 64 KB.
+    // takes 16 KB of its own from the front of the rings.
     asm volatile("s_barrier" ::: "memory");
     uint8_t* bounce = lds + wv * 16384 + lane2 * 16;
     const uint32_t bounce_at = uint32_t(uintptr_t((lds_ptr)bounce));
@@ -363,16 +387,16 @@ __device__ __forceinline__ void fc1_tile_body(const Fc1Args& a, const Chunk ch, 
 // FC2 for chunk c by one workgroup: 256 output columns x 16*TT rows; the wave owns block ob.
 // `verdict` is rowbad[c][lane % 16] (bit 8+t: tile t holds a token in this row), fetched by the caller beside
 // the chunk record.
-template <int TT>
+template <class S, int TT>
 __device__ __forceinline__ void fc2_tile_body(const Fc2Args& a, const Chunk ch, uint32_t c, uint32_t ob, uint32_t wv,
                                               uint32_t lane, uint8_t* lds, const uint32_t verdict) {
-    constexpr int kMine = TT / kTileWaves;
+    constexpr int kMine = staged_tiles<S, TT>();
     const uint32_t r = lane & 15, g = lane >> 4, I = a.lay.inter;
     const int32_t expert = ch.expert;
     const uint8_t* row[kMine];
 #pragma unroll
     for (int m = 0; m < kMine; ++m) {
-        const int lt = int(wv) * kMine + m;
+        const int lt = int(first_staged_tile<S, TT>(wv)) + m;
         const bool mine = (verdict >> (8 + lt)) & 1u;
         const size_t grow = size_t(ch.first_group + lt) * 16 + r;
         row[m] = (mine ? a.dq + grow * I : a.zero_row) + g * 16;
@@ -387,14 +411,14 @@ __device__ __forceinline__ void fc2_tile_body(const Fc2Args& a, const Chunk ch, 
     for (int t = 0; t < 4; ++t)
 #pragma unroll
         for (int tt = 0; tt < TT; ++tt) acc[t][tt] = v4f{0.f, 0.f, 0.f, 0.f};
-    gemm_chunk_lds<TT>(acc, wp, sp, sx, int(ksteps), row, wv, lane, lds);
+    gemm_chunk_lds<S, TT>(acc, wp, sp, sx, int(ksteps), row, wv, lane, lds);
     const uint32_t lane2 = after_loop(lane);
     // A lane holds four consecutive output columns of one token per tile, so a store straight from the
     // accumulators touches sixteen token rows with 64 bytes each. One trip through the wave's own, now
     // idle, weight ring regroups a tile row into 256 contiguous bytes per token (sixteen lanes) and
     // four tokens per store: a tenth off the kernel at 8192 tokens. Cells are 272 bytes apart so the
     // regrouped reads (same token, sixteen cells) fall on different banks.
-    uint8_t* ring = lds + wv * (kWeightStages * 4096);
+    uint8_t* ring = lds + wv * (S::kWeightStages * 4096);
     const uint32_t cell = lane2 & 15, token4 = lane2 >> 4;  // regrouped: sixteen 16-byte cells of one token, four tokens
     const uint32_t put_at = uint32_t(uintptr_t((lds_ptr)ring)) + (lane2 >> 4) * 272 + (lane2 & 15) * 16;
     bool lost = false;
@@ -438,19 +462,24 @@ __host__ inline uint32_t tile_grid(uint32_t columns, uint32_t chunk_cap) {
     return columns * ((chunk_cap + 8 * kTileRun - 1) / (8 * kTileRun) * (8 * kTileRun));
 }
 
-// 256 threads, one workgroup per (chunk, 128 intermediate columns). Chunks of one or two groups run
-// the register-only bodies (each wave is independent there); larger chunks share activations
+// One workgroup of S::kWaves waves per (chunk, 32 * kWaves intermediate columns). Chunks of one or two groups
+// run the register-only bodies (each wave is independent there); larger chunks share activations
 // through LDS.
-__global__ void __launch_bounds__(kTileThreads, 2) fc1_tile_kernel(Fc1Args a) {
+template <class S>
+__global__ void __launch_bounds__(S::kThreads, 8 / S::kWaves) fc1_tile_kernel(Fc1Args a) {
     extern __shared__ __align__(16) uint8_t lds[];
     uint32_t* meta = a.plan.meta;
-    const TileItem it = tile_item(a.lay.inter / 128);
+    const TileItem it = tile_item(a.lay.inter / (32 * S::kWaves));
     const uint32_t c = it.chunk;
-    const uint32_t lane = threadIdx.x & 63, wv = threadIdx.x >> 6, cb = it.column * 4 + wv;
-    // The row table's entries this lane may need (tile wv when the chunk runs as four tiles, tiles 2wv and
-    // 2wv+1 as eight), asked for beside the record: the table covers the whole grid.
+    const uint32_t lane = threadIdx.x & 63, wv = threadIdx.x >> 6, cb = it.column * S::kWaves + wv;
+    // The row table's entries this lane may need, as four tiles and as eight, asked for beside the record:
+    // the table covers the whole grid.
     const int32_t* xr = a.xrows + size_t(c) * 128 + (lane & 15);
-    const int32_t token4 = xr[wv * 16], token8[2] = {xr[(2 * wv) * 16], xr[(2 * wv + 1) * 16]};
+    int32_t token4[staged_tiles<S, 4>()], token8[staged_tiles<S, 8>()];
+#pragma unroll
+    for (int m = 0; m < staged_tiles<S, 4>(); ++m) token4[m] = xr[(first_staged_tile<S, 4>(wv) + m) * 16];
+#pragma unroll
+    for (int m = 0; m < staged_tiles<S, 8>(); ++m) token8[m] = xr[(first_staged_tile<S, 8>(wv) + m) * 16];
     const ItemHead head = load_item_head(a.plan.chunks + c, meta);  // the chunk table covers the whole grid too
     const Chunk ch = head.ch;
     if (head.meta[kPlanFault] || c >= head.meta[kChunkCount]) return;
@@ -461,17 +490,18 @@ __global__ void __launch_bounds__(kTileThreads, 2) fc1_tile_kernel(Fc1Args a) {
     }
     if (ch.groups == 1) fc1_body<1>(a, ch, cb, lane);
     else if (ch.groups == 2) fc1_body<2>(a, ch, cb, lane);
-    else if (ch.groups <= 4) fc1_tile_body<4>(a, ch, c, cb, wv, lane, lds, {token4});
-    else fc1_tile_body<8>(a, ch, c, cb, wv, lane, lds, token8);
+    else if (ch.groups <= 4) fc1_tile_body<S, 4>(a, ch, c, cb, wv, lane, lds, token4);
+    else fc1_tile_body<S, 8>(a, ch, c, cb, wv, lane, lds, token8);
 }
 
-// 256 threads, one workgroup per (chunk, 256 output columns).
-__global__ void __launch_bounds__(kTileThreads, 2) fc2_tile_kernel(Fc2Args a) {
+// One workgroup per (chunk, 64 * kWaves output columns).
+template <class S>
+__global__ void __launch_bounds__(S::kThreads, 8 / S::kWaves) fc2_tile_kernel(Fc2Args a) {
     extern __shared__ __align__(16) uint8_t lds[];
     uint32_t* meta = a.plan.meta;
-    const TileItem it = tile_item(kHidden / 256);
+    const TileItem it = tile_item(kHidden / (64 * S::kWaves));
     const uint32_t c = it.chunk;
-    const uint32_t lane = threadIdx.x & 63, wv = threadIdx.x >> 6, ob = it.column * 4 + wv;
+    const uint32_t lane = threadIdx.x & 63, wv = threadIdx.x >> 6, ob = it.column * S::kWaves + wv;
     const uint32_t verdict = a.rowbad[c * 16 + (lane & 15)];  // beside the record: the table covers the whole grid
     const ItemHead head = load_item_head(a.plan.chunks + c, meta);
     const Chunk ch = head.ch;
@@ -483,8 +513,10 @@ __global__ void __launch_bounds__(kTileThreads, 2) fc2_tile_kernel(Fc2Args a) {
     }
     if (ch.groups == 1) fc2_body<1>(a, ch, ob, lane);
     else if (ch.groups == 2) fc2_body<2>(a, ch, ob, lane);
-    else if (ch.groups <= 4) fc2_tile_body<4>(a, ch, c, ob, wv, lane, lds, verdict);
-    else fc2_tile_body<8>(a, ch, c, ob, wv, lane, lds, verdict);
+#ifndef EXP_FC2_ALL8
+    else if (ch.groups <= 4) fc2_tile_body<S, 4>(a, ch, c, ob, wv, lane, lds, verdict);
+#endif
+    else fc2_tile_body<S, 8>(a, ch, c, ob, wv, lane, lds, verdict);
 }
 
 }  // namespace m26g

@@ -209,6 +209,29 @@ def test_decode_layer_full_intermediate(scratch, full_layer):
     check_stages(scratch, layer, wl, pools, stats)
 
 
+def test_tile_schedule_at_full_intermediate_every_row(scratch, full_layer):
+    """The prefill schedule at I = 2048, where FC2 runs several quads of k-steps: a few experts under skewed
+    routing so that chunks of three and four groups (the four-tile bodies, last tile in use) and of five to
+    eight occur, every row against the CPU reference and two runs bit for bit. (With one quad, as at one
+    rank's share, the k-loop is not a loop, and what the compiler places behind a loop's last MFMA never runs.)"""
+    _, pools, layer = full_layer
+    seed, rows = synth.BASE_SEED + 13, 312
+    experts = list(range(5, 256, 21))  # 12 experts
+    ids, w, x = _skewed_routes(seed, rows, experts), synth._softmax_weights(seed, rows), synth._activations(seed, rows)
+    groups_of = (np.bincount(ids.reshape(-1), minlength=256) + 15) // 16
+    assert (groups_of % 8 == 4).any() and (groups_of % 8 == 3).any() and (groups_of >= 5).any(), groups_of[groups_of > 0]
+    payload, scales = synth.q0_quantize(x)
+    wl = synth.Workload("tile schedule, full intermediate", 3, seed, 4, rows, ids, w, x, payload, scales)
+    stats, bf, pf = run_ffn_dev(layer, scratch, wl)
+    rc, ref_partial, ref_bf16, _ = O.layer_ffn(pools, wl.payload, wl.scales, wl.ids, wl.weights)
+    assert rc == 0
+    check_outputs(pf, bf, ref_partial, ref_bf16)
+    per_row = np.abs(pf - ref_partial).max(axis=1) / np.abs(ref_partial).max()
+    assert per_row.max() <= MAX_ABS, ("worst row", int(per_row.argmax()), float(per_row.max()))
+    _, bf2, pf2 = run_ffn_dev(layer, scratch, wl)
+    assert np.array_equal(bf2, bf) and np.array_equal(pf2.view(np.uint32), pf.view(np.uint32))
+
+
 def test_prefill_chunk_properties_and_sampled_parity(full_layer):
     """configs[3] at its full 8192 tokens: 48 sampled rows against the CPU reference, and size-independent
     properties over all rows: each row depends on its own routes only (a subset run alone reproduces
@@ -234,6 +257,8 @@ def test_prefill_chunk_properties_and_sampled_parity(full_layer):
     rc, ref_partial, ref_bf16, _ = O.layer_ffn(pools, sub.payload, sub.scales, sub.ids, sub.weights)
     assert rc == 0
     check_outputs(pf[sample], bf[sample], ref_partial, ref_bf16)
+    _, bf_again, pf_again = run_ffn_dev(layer, s, wl)                     # every row, bit for bit, run after run
+    assert np.array_equal(bf_again, bf) and np.array_equal(pf_again.view(np.uint32), pf.view(np.uint32))
     _, bf_sub, pf_sub = run_ffn_dev(layer, s, sub)
     assert np.array_equal(bf_sub, bf[sample]) and np.array_equal(pf_sub.view(np.uint32), pf[sample].view(np.uint32))
     perm = np.random.default_rng(1).permutation(wl.rows)
