@@ -124,7 +124,7 @@ Workspace carve(uint8_t* base, const Shape& s) {
     const uint64_t I = s.inter, gcap = w.group_cap, ccap = w.chunk_cap;
     // The tile kernels ask for their chunk record, row table and row verdicts before they know whether the
     // chunk exists: those tables cover the whole grid (chunk capacity rounded up to runs on eight XCDs).
-    const uint64_t grid_chunks = ccap + 8 * kTileRun;
+    const uint64_t grid_chunks = ccap + 8 * kTileRunMax;
     w.plan_work = reinterpret_cast<uint32_t*>(take(kPlanWorkBytes));
     w.inverse = reinterpret_cast<int32_t*>(take(w.bytes[0] = w.route_cap * 4));
     w.original = reinterpret_cast<int32_t*>(take(w.bytes[1] = w.route_cap * 4));
@@ -159,11 +159,7 @@ Workspace carve(uint8_t* base, const Shape& s) {
 
 // Kernels whose dynamic LDS passes 64 KB need the limit raised once per process.
 bool lds_ready = false;
-#ifdef EXP_TILE8
-using TileS = Tile8;
-#else
-using TileS = Tile4;
-#endif
+using TileS = PrefillTile;
 hipError_t raise_lds_limits() {
     if (lds_ready) return hipSuccess;
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(plan_kernel),
@@ -307,9 +303,9 @@ void launch_direct(const m26s_b1_layer* L, const Launch& k, const Fc1Args& f1, c
 void launch_tiles(const m26s_b1_layer* L, const Launch& k, const Fc1Args& f1, const Fc2Args& f2) {
     gather_scales_kernel<<<k.ws.chunk_cap, 256, 0, k.stream>>>(f1.plan, f1.xs, f1.xs_pitch, reinterpret_cast<uint32_t*>(k.ws.xg),
                                                               k.ws.rowbad, k.ws.xrows, k.ws.yrows);
-    fc1_tile_kernel<TileS><<<tile_grid(L->lay.inter / (32 * TileS::kWaves), k.ws.chunk_cap), TileS::kThreads, TileS::kLdsBytes, k.stream>>>(f1);
+    fc1_tile_kernel<TileS><<<tile_grid(L->lay.inter / (32 * TileS::kWaves), k.ws.chunk_cap, kFc1Run), TileS::kThreads, TileS::kLdsBytes, k.stream>>>(f1);
     mark(k.fc1_done, k.stream);
-    fc2_tile_kernel<TileS><<<tile_grid(kHidden / (64 * TileS::kWaves), k.ws.chunk_cap), TileS::kThreads, TileS::kLdsBytes, k.stream>>>(f2);
+    fc2_tile_kernel<TileS><<<tile_grid(kHidden / (64 * TileS::kWaves), k.ws.chunk_cap, kFc2Run), TileS::kThreads, TileS::kLdsBytes, k.stream>>>(f2);
     mark(k.fc2_done, k.stream);
 }
 // Layers with exceptional weight scales: decode-then-multiply, group by group.

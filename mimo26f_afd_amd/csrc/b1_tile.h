@@ -1,17 +1,17 @@
-// Prefill-size schedule of FC1 / FC2: workgroups of four waves, two workgroups per compute unit.
+// Prefill-size schedule of FC1 / FC2: one workgroup of eight waves per compute unit.
 //
 // A wave accumulates one column block (four weight tiles: 32 intermediate columns of FC1, 64 output
 // columns of FC2) against all TT activation tiles of its chunk: 4*TT accumulator tiles, 128
-// accumulation registers at TT = 8, which leaves the other half of the register file to a second
-// workgroup on the same SIMDs. That second workgroup is what hides everything that is not an MFMA:
-// while one workgroup looks up its chunk, waits for its first operands or runs its epilogue
-// (SwiGLU + requantisation, or the FP32 row stores), the other one multiplies.
+// accumulation registers at TT = 8, half of the register file of a wave at two waves per SIMD. The two
+// waves of a SIMD belong to the same workgroup and run the same k-step; each fills the issue gaps of
+// the other (a wave's own loads and LDS reads hold its in-order issue for longer than an MFMA's
+// shadow).
 //
 // Operands travel global -> LDS with the direct-to-LDS loads of gfx950 (no staging registers, so the
-// prefetch depth is paid in LDS, not in VGPRs), always two k-steps ahead of the MFMAs that consume
-// them: every wave streams its own weight fragments into a private two-stage ring (a stage is free
+// prefetch depth is paid in LDS, not in VGPRs), always three k-steps ahead of the MFMAs that consume
+// them: every wave streams its own weight fragments into a private three-stage ring (a stage is free
 // once its fragments sit in registers), and the chunk's activation tiles are staged once per
-// workgroup in a three-stage ring shared by the four waves. Scales never touch LDS: weight scales
+// workgroup in a four-stage ring shared by the eight waves. Scales never touch LDS: weight scales
 // are stored in MFMA lane order by the one-time preparation, and activation scales are brought into
 // the same order per chunk (gather_scales_kernel for the caller's rows, the FC1 epilogue for the
 // intermediate), so one dword per lane carries the scale bytes of four k-steps and the MFMA picks
@@ -20,8 +20,8 @@
 // Reference counterparts: fc1_m64 / fc2_m64, the weight-reuse chunk kernels of
 // crates/mimo26-spark/kernels/b1_fc1_m64.cuh:111-205,378-491 (cp.async multi-stage staging there).
 //
-// LDS, dynamic, 80 KB:  [4 waves][2 stages][4 tiles][64 lanes][16 B]   weight fragments (private per wave)
-//                       [3 stages][8 tiles][2 halves][64 lanes][16 B]  activation fragments (shared)
+// LDS, dynamic, 160 KB: [8 waves][3 stages][4 tiles][64 lanes][16 B]   weight fragments (private per wave)
+//                       [4 stages][8 tiles][2 halves][64 lanes][16 B]  activation fragments (shared)
 // All fragment cells sit in MFMA lane order, so one direct load fills a 1 KB cell row and one
 // ds_read_b128 per lane reads it back without bank conflicts. The compiler does not order LDS reads
 // against direct-to-LDS loads; the vmcnt waits below do, and rely on the issue order stated there.
@@ -41,9 +41,13 @@ struct TileShape {
     static constexpr int kWaves = W, kAhead = D, kThreads = 64 * W, kWeightStages = D, kActStages = D + 1;
     static constexpr uint32_t kLdsBytes = W * D * 4096 + (D + 1) * 8 * 2048;
 };
-using Tile4 = TileShape<4, 2>;  // 80 KB: two workgroups per compute unit
-using Tile8 = TileShape<8, 3>;  // 160 KB: one workgroup per compute unit, rows shared by eight waves
-static_assert(Tile4::kLdsBytes == 80 * 1024 && Tile8::kLdsBytes == 160 * 1024, "the 160 KB of a compute unit");
+// Eight waves, three k-steps ahead: the whole LDS of a compute unit for one workgroup. Against four waves two
+// steps ahead, two workgroups per compute unit (80 KB each, what this schedule was first built as), a chunk's rows
+// enter the compute unit once instead of twice (48 instead of 64 KB per k-step) and the saved LDS buys the third
+// step of prefetch: measured on one box 4 % off FC1 and 6.4 % off FC2 at 8192 tokens, ahead from 256 rows up,
+// level at 192, 2 % behind at 130.
+using PrefillTile = TileShape<8, 3>;
+static_assert(PrefillTile::kLdsBytes == 160 * 1024, "the 160 KB of a compute unit");
 // Bytes of one chunk's gathered activation scales for a K-deep product: [K/512][8][64] dwords.
 __host__ __device__ constexpr uint32_t gathered_scale_bytes(uint32_t k) { return (k / 512) * 2048; }
 
@@ -211,10 +215,6 @@ __device__ __forceinline__ void gemm_chunk_lds(v4f (&acc)[4][TT], const uint8_t*
     lds_barrier();
     v4i flo, fhi;  // the fragment a k-step starts with
     read_fragment(flo, fhi, aring_at);
-    // While it multiplies, the wave outranks the other workgroup's wave on its SIMD, whose set-up or
-    // epilogue instructions otherwise take issue slots from this loop's fragment reads and loads
-    // (measured: 2 % off FC1 at 8192 tokens).
-    __builtin_amdgcn_s_setprio(3);
     uint32_t wr = 0, ar = 0;  // weight stage of step k, which takes step k+kAhead; activation stage of step k
     int q = 0;
     // One k-step with MFMA scale select b = ks % 4 (an immediate, hence the macro).
@@ -244,8 +244,10 @@ __device__ __forceinline__ void gemm_chunk_lds(v4f (&acc)[4][TT], const uint8_t*
                     if (item * TT / kPerStep == tt) stage_item(item, ahead, ar2, wr);                          \
                 __builtin_amdgcn_sched_barrier(0);                                                             \
                 /* Everything but the loads of the last kAhead-1 steps has landed: activations and     */      \
-                /* weights of step k+1, and the next quad's scales, older still.                        */      \
-                wait_loads_but<(kAhead - 1) * kPerStep>();                                                     \
+                /* weights of step k+1. The next quad's scales were asked for at the head of step 0,    */      \
+                /* behind the loads of the step before: with more than one step in flight they lie      */      \
+                /* inside that window, and step 0 leaves them in flight too.                            */      \
+                wait_loads_but<(kAhead - 1) * kPerStep + ((b) == 0 && kAhead > 2 ? 4 + TT : 0)>();              \
                 lds_barrier(); /* with the wait for this group's fragment */                                   \
                 read_fragment(flo, fhi, aring_at + ar1 * TT * 2048);                                           \
                 read_weights(af[((b) + 1) & 1], wr1);                                                          \
@@ -300,7 +302,6 @@ __device__ __forceinline__ void gemm_chunk_lds(v4f (&acc)[4][TT], const uint8_t*
     if (q < quads) M26G_QUAD(sw0, sa0, sw1, sa1)  // odd count: an even number of quads ends on set 0
 #undef M26G_QUAD
 #undef M26G_KSTEP
-    __builtin_amdgcn_s_setprio(0);
     wait_loads_but<0>();  // the re-staged tail loads must land before the LDS is reused or the wave ends
     wait_lds_but<0>();
     // The last fetches of scales, fragment and weights feed no MFMA. To the compiler such a register is
@@ -355,7 +356,7 @@ __device__ __forceinline__ void fc1_tile_body(const Fc1Args& a, const Chunk ch, 
     // The accumulators leave the accumulation registers through LDS, sixteen tiles at a time: whole-tile
     // writes keep them out of the register allocator's hands until the very end (element reads straight
     // from the accumulation file make it split their live ranges across the k-loop), and the epilogue
-    // becomes one rolled loop over the activation tiles. Unrolled it is 70 KB of code, and two workgroups
+    // becomes one rolled loop over the activation tiles. Unrolled it is 70 KB of code, and workgroups
     // in different phases then evict each other's instructions from the cache the compute units share.
     // Every wave has drained its own direct loads; after the barrier nobody's are left, and each wave
     // takes 16 KB of its own from the front of the rings.
@@ -447,19 +448,22 @@ __device__ __forceinline__ void fc2_tile_body(const Fc2Args& a, const Chunk ch, 
 
 // Work item of a tile workgroup. Workgroups are handed to the eight XCDs in turn, each with an L2 of
 // its own: the `columns` workgroups of one chunk all take ids of one residue mod 8, so a chunk's
-// activation rows enter one L2 only, and so do those of the chunk after it: chunks are in expert
-// order, two neighbours mostly share their expert, and their workgroups of one column, dispatched
-// back to back, stream the same weights through that L2 (measured: 2.7 % off FC1 at 8192 tokens; runs
-// of four gained less). The grid is columns * (chunk capacity rounded up to 8 runs).
+// activation rows enter one L2 only. FC2 hands an XCD runs of two neighbouring chunks: chunks are in
+// expert order, two neighbours mostly share their expert, and their workgroups of one column, dispatched
+// back to back, stream the same weights through that L2. Measured with eight-wave workgroups at 8192
+// tokens: runs of two against single chunks take 1.4 % off FC2 and add 1.8 % to FC1 (whose workgroup
+// streams four times the weight bytes per chunk and shares less of its time with its neighbour); runs of
+// four lose 2 % and 5 %. The grid is columns * (chunk capacity rounded up to 8 runs).
 struct TileItem { uint32_t chunk, column; };
-constexpr uint32_t kTileRun = 2;  // neighbouring chunks per XCD
+constexpr uint32_t kFc1Run = 1, kFc2Run = 2, kTileRunMax = 2;  // neighbouring chunks per XCD
+template <uint32_t RUN>
 __device__ __forceinline__ TileItem tile_item(uint32_t columns) {
     const uint32_t id = blockIdx.x, xcd = id & 7, slot = id >> 3;
-    const uint32_t per = columns * kTileRun, run = slot / per, within = slot % per;
-    return TileItem{(run * 8 + xcd) * kTileRun + within % kTileRun, within / kTileRun};
+    const uint32_t per = columns * RUN, run = slot / per, within = slot % per;
+    return TileItem{(run * 8 + xcd) * RUN + within % RUN, within / RUN};
 }
-__host__ inline uint32_t tile_grid(uint32_t columns, uint32_t chunk_cap) {
-    return columns * ((chunk_cap + 8 * kTileRun - 1) / (8 * kTileRun) * (8 * kTileRun));
+__host__ inline uint32_t tile_grid(uint32_t columns, uint32_t chunk_cap, uint32_t run) {
+    return columns * ((chunk_cap + 8 * run - 1) / (8 * run) * (8 * run));
 }
 
 // One workgroup of S::kWaves waves per (chunk, 32 * kWaves intermediate columns). Chunks of one or two groups
@@ -469,7 +473,7 @@ template <class S>
 __global__ void __launch_bounds__(S::kThreads, 8 / S::kWaves) fc1_tile_kernel(Fc1Args a) {
     extern __shared__ __align__(16) uint8_t lds[];
     uint32_t* meta = a.plan.meta;
-    const TileItem it = tile_item(a.lay.inter / (32 * S::kWaves));
+    const TileItem it = tile_item<kFc1Run>(a.lay.inter / (32 * S::kWaves));
     const uint32_t c = it.chunk;
     const uint32_t lane = threadIdx.x & 63, wv = threadIdx.x >> 6, cb = it.column * S::kWaves + wv;
     // The row table's entries this lane may need, as four tiles and as eight, asked for beside the record:
@@ -499,7 +503,7 @@ template <class S>
 __global__ void __launch_bounds__(S::kThreads, 8 / S::kWaves) fc2_tile_kernel(Fc2Args a) {
     extern __shared__ __align__(16) uint8_t lds[];
     uint32_t* meta = a.plan.meta;
-    const TileItem it = tile_item(kHidden / (64 * S::kWaves));
+    const TileItem it = tile_item<kFc2Run>(kHidden / (64 * S::kWaves));
     const uint32_t c = it.chunk;
     const uint32_t lane = threadIdx.x & 63, wv = threadIdx.x >> 6, ob = it.column * S::kWaves + wv;
     const uint32_t verdict = a.rowbad[c * 16 + (lane & 15)];  // beside the record: the table covers the whole grid
@@ -513,9 +517,7 @@ __global__ void __launch_bounds__(S::kThreads, 8 / S::kWaves) fc2_tile_kernel(Fc
     }
     if (ch.groups == 1) fc2_body<1>(a, ch, ob, lane);
     else if (ch.groups == 2) fc2_body<2>(a, ch, ob, lane);
-#ifndef EXP_FC2_ALL8
     else if (ch.groups <= 4) fc2_tile_body<S, 4>(a, ch, c, ob, wv, lane, lds, verdict);
-#endif
     else fc2_tile_body<S, 8>(a, ch, c, ob, wv, lane, lds, verdict);
 }
 
