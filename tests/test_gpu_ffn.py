@@ -233,7 +233,7 @@ def test_tile_schedule_at_full_intermediate_every_row(scratch, full_layer):
 
 
 def test_prefill_chunk_properties_and_sampled_parity(full_layer):
-    """configs[3] at its full 8192 tokens: 48 sampled rows against the CPU reference, and size-independent
+    """configs[3] at its full 8192 tokens: some 390 sampled rows against the CPU reference, and size-independent
     properties over all rows: each row depends on its own routes only (a subset run alone reproduces
     its rows bit for bit, a permuted batch permutes the rows), and the plan is a stable bijection."""
     _, pools, layer = full_layer  # the same seeded weights serve both configurations
@@ -251,7 +251,7 @@ def test_prefill_chunk_properties_and_sampled_parity(full_layer):
     assert np.all(np.diff(experts) >= 0)
     same = np.diff(experts) == 0
     assert np.all(np.diff(orig)[same] > 0)                                 # stable inside every expert
-    sample = np.unique(np.concatenate([[0, 1, 777, 4095, 4096, 8191], np.random.default_rng(3).integers(0, wl.rows, 42)]))
+    sample = np.unique(np.concatenate([[0, 1, 777, 4095, 4096, 8191], np.random.default_rng(3).integers(0, wl.rows, 394)]))
     sub = synth.Workload("sample", 3, wl.seed, 4, len(sample), wl.ids[sample], wl.weights[sample], wl.x[sample],
                          wl.payload[sample], wl.scales[sample])
     rc, ref_partial, ref_bf16, _ = O.layer_ffn(pools, sub.payload, sub.scales, sub.ids, sub.weights)
