@@ -15,8 +15,8 @@ and this module checks them on the assembly hipcc emits (no GPU needed):
     right behind the last MFMA of a loop (to hand the accumulator to the code after the loop in another
     register) reads the value from before that MFMA. The sources put `s_nop` runs where such code can
     follow; the check counts wait states (one per instruction, N + 1 for `s_nop N`) between a
-    hand-written MFMA and the next non-MFMA access to its destination, and wants at least 12
-    (8 passes + 3, the figure the compiler's own hazard tables hold for this MFMA, and one to spare).
+    hand-written MFMA and the next non-MFMA access to its destination, and wants at least 16
+    (the compiler's own hazard tables hold 8 passes + 3 for this MFMA; the rest is margin).
 
 "In flight" follows the hardware's counters. Vector-memory operations (loads, stores, direct-to-LDS
 loads, whoever issued them) complete in issue order, and `s_waitcnt vmcnt(N)` returns when at most N
@@ -45,7 +45,7 @@ NO_DEST = ("global_load_lds", "global_store", "ds_write", "v_readfirstlane", "v_
            "scratch_store", "global_atomic")
 
 
-MFMA_WAIT_STATES = 12
+MFMA_WAIT_STATES = 16
 
 
 def _aregs(tok: str) -> set:

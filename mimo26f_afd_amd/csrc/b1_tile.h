@@ -290,8 +290,8 @@ __device__ __forceinline__ void gemm_chunk_lds(v4f (&acc)[4][TT], const uint8_t*
         M26G_KSTEP(3, SW, SA)                                                                                  \
         /* The compiler may put anything behind a quad, a copy of an accumulator included (it hands them to */ \
         /* the code after the loop in other registers when it likes), and it does not know that the last  */ \
-        /* MFMA's result is eight passes away: twelve wait states cover that.                             */ \
-        asm volatile("s_nop 11" ::: "memory");                                                                \
+        /* MFMA's result is eight passes away: sixteen wait states cover that with room to spare.         */ \
+        asm volatile("s_nop 15" ::: "memory");                                                                \
         ++q;                                                                                                   \
     }
 #pragma unroll 1

@@ -55,23 +55,23 @@ def test_checker_retires_vector_memory_operations_in_issue_order():
 def test_checker_keeps_everything_but_mfmas_off_a_fresh_accumulator():
     """A hand-written MFMA's result is eight passes away and the compiler does not know: an accumulator copy
     or read it places right behind one (as it does behind a loop, to hand the accumulator on in another
-    register) is a hazard until twelve wait states have passed; another MFMA on the same accumulator is not."""
+    register) is a hazard until sixteen wait states have passed; another MFMA on the same accumulator is not."""
     mfma = hand("v_mfma_scale_f32_16x16x128_f8f6f4 a[64:67], v[10:13], v[20:27], a[64:67], v7, v8 op_sel_hi:[0,0,0] cbsz:4")
     copy = "\tv_accvgpr_mov_b32 a60, a64"
     _, p = codegen_check.check(asm(mfma, "\ts_add_i32 s35, s35, 3", copy))
     assert len(p) == 1 and "accumulator" in p[0]
-    _, p = codegen_check.check(asm(mfma, hand("s_nop 11"), copy))
+    _, p = codegen_check.check(asm(mfma, hand("s_nop 15"), copy))
     assert p == []
-    _, p = codegen_check.check(asm(mfma, hand("s_nop 9"), copy))           # ten wait states and the copy's own slot: too few
+    _, p = codegen_check.check(asm(mfma, hand("s_nop 13"), copy))          # fourteen wait states: too few
     assert len(p) == 1
-    _, p = codegen_check.check(asm(mfma, mfma, hand("s_nop 11"), "\tv_accvgpr_read_b32 v1, a65"))
+    _, p = codegen_check.check(asm(mfma, mfma, hand("s_nop 15"), "\tv_accvgpr_read_b32 v1, a65"))
     assert p == []
     _, p = codegen_check.check(asm(mfma, hand("ds_write_b128 v3, a[64:67] offset:1024")))
     assert len(p) == 1
     # behind a loop: the exit block is reached from the loop's last MFMA whatever lies between them in the file
     _, p = codegen_check.check(asm(".LBB0_1:", mfma, "\ts_cbranch_scc1 .LBB0_1", copy, "\ts_endpgm"))
     assert len(p) == 1
-    _, p = codegen_check.check(asm(".LBB0_1:", mfma, hand("s_nop 11"), "\ts_cbranch_scc1 .LBB0_1", copy, "\ts_endpgm"))
+    _, p = codegen_check.check(asm(".LBB0_1:", mfma, hand("s_nop 15"), "\ts_cbranch_scc1 .LBB0_1", copy, "\ts_endpgm"))
     assert p == []
 
 
