@@ -265,7 +265,7 @@ def compile_to_asm() -> str:
 def run() -> dict:
     """Compile, check, raise on any problem; returns the per-kernel count of hand-issued loads."""
     seen, problems = check(compile_to_asm())
-    if len(seen) < 2 or min(seen.values()) < 100:
+    if len(seen) < 3 or min(seen.values()) < 100:
         raise RuntimeError(f"codegen check: tile kernels not found in the assembly ({seen})")
     if problems:
         raise RuntimeError("codegen check failed:\n" + "\n".join(problems[:12]))

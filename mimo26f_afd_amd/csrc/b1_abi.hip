@@ -168,7 +168,10 @@ hipError_t raise_lds_limits() {
         e = hipFuncSetAttribute(reinterpret_cast<const void*>(fc1_tile_kernel<TileS>),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, int(TileS::kLdsBytes));
     if (e == hipSuccess)
-        e = hipFuncSetAttribute(reinterpret_cast<const void*>(fc2_tile_kernel<TileS>),
+        e = hipFuncSetAttribute(reinterpret_cast<const void*>(fc2_tile_kernel<TileS, false>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, int(TileS::kLdsBytes));
+    if (e == hipSuccess)
+        e = hipFuncSetAttribute(reinterpret_cast<const void*>(fc2_tile_kernel<TileS, true>),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, int(TileS::kLdsBytes));
     lds_ready = e == hipSuccess;
     return e;
@@ -305,7 +308,9 @@ void launch_tiles(const m26s_b1_layer* L, const Launch& k, const Fc1Args& f1, co
                                                               k.ws.rowbad, k.ws.xrows, k.ws.yrows);
     fc1_tile_kernel<TileS><<<tile_grid(L->lay.inter / (32 * TileS::kWaves), k.ws.chunk_cap, kFc1Run), TileS::kThreads, TileS::kLdsBytes, k.stream>>>(f1);
     mark(k.fc1_done, k.stream);
-    fc2_tile_kernel<TileS><<<tile_grid(kHidden / (64 * TileS::kWaves), k.ws.chunk_cap, kFc2Run), TileS::kThreads, TileS::kLdsBytes, k.stream>>>(f2);
+    const dim3 grid2(tile_grid(kHidden / (64 * TileS::kWaves), k.ws.chunk_cap, kFc2Run));
+    if (L->lay.inter == kRankI) fc2_tile_kernel<TileS, true><<<grid2, TileS::kThreads, TileS::kLdsBytes, k.stream>>>(f2);
+    else fc2_tile_kernel<TileS, false><<<grid2, TileS::kThreads, TileS::kLdsBytes, k.stream>>>(f2);
     mark(k.fc2_done, k.stream);
 }
 // Layers with exceptional weight scales: decode-then-multiply, group by group.

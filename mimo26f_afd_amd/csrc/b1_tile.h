@@ -147,7 +147,9 @@ __global__ void __launch_bounds__(256) gather_scales_kernel(PlanView plan, const
 // per k-step: `row[i]` is this lane's row of tile wv*(TT/4)+i (lane offset 16*(lane/16) included),
 // so the lane that loads a fragment cell is the lane that will hold it. `sx` points at this lane's
 // dword of tile 0, quad 0 of the chunk's gathered activation scales.
-template <class S, int TT>
+// ONE: the product is a single quad of k-steps deep (FC2 at one rank's share); otherwise the number of quads is
+// even (8 for FC1, 4 for FC2 of a whole layer), which fixes the scale set the last quad runs on.
+template <class S, int TT, bool ONE>
 __device__ __forceinline__ void gemm_chunk_lds(v4f (&acc)[4][TT], const uint8_t* __restrict__ wp,
                                                const uint8_t* __restrict__ sp, const uint8_t* __restrict__ sx, int ksteps,
                                                const uint8_t* const (&row)[(2 * TT / S::kWaves + 1) / 2], uint32_t wv,
@@ -225,7 +227,7 @@ __device__ __forceinline__ void gemm_chunk_lds(v4f (&acc)[4][TT], const uint8_t*
     // waits for them. The workgroup barrier sits ahead of the last group's MFMAs, not behind them: what
     // it orders (every wave's loads of step k+1 landed, every wave's reads of step k done) is true by
     // then, and the first fragment of step k+1 and the next weights are fetched under those MFMAs.
-#define M26G_KSTEP(b, SW, SA)                                                                                  \
+#define M26G_KSTEP(b, SW, SA, STAGE, ALLOW, NEXT)                                                              \
     {                                                                                                          \
         const int ks = 4 * q + (b);                                                                            \
         /* Weights of step k sit in registers, so their stage `wr` takes step k+kAhead; step k+1 is   */      \
@@ -233,24 +235,27 @@ __device__ __forceinline__ void gemm_chunk_lds(v4f (&acc)[4][TT], const uint8_t*
         /* step k+kAhead goes to the stage before ar, which step k-1 has finished with.               */      \
         const uint32_t ar1 = ar == kActStages - 1 ? 0 : ar + 1, ar2 = ar == 0 ? kActStages - 1 : ar - 1;       \
         const uint32_t wr1 = wr == kWeightStages - 1 ? 0 : wr + 1;                                             \
-        /* Past the end the last step is staged again into stages nobody reads any more. */                   \
-        const int ahead = ks + kAhead < last ? ks + kAhead : last;                                             \
+        const int ahead = ks + kAhead; /* the step staged under this one (STAGE: it exists) */               \
         const uint32_t fs = aring_at + ar * TT * 2048;                                                         \
         v4i lo = flo, hi = fhi; /* fragment 0, fetched at the end of the step before */                       \
         _Pragma("unroll") for (int tt = 0; tt < TT; ++tt) {                                                    \
             v4i nlo = lo, nhi = hi;                                                                            \
             if (tt == TT - 1) {                                                                                \
-                _Pragma("unroll") for (int item = 0; item < kPerStep; ++item)                                  \
-                    if (item * TT / kPerStep == tt) stage_item(item, ahead, ar2, wr);                          \
+                if (STAGE) {                                                                                   \
+                    _Pragma("unroll") for (int item = 0; item < kPerStep; ++item)                              \
+                        if (item * TT / kPerStep == tt) stage_item(item, ahead, ar2, wr);                      \
+                }                                                                                              \
                 __builtin_amdgcn_sched_barrier(0);                                                             \
-                /* Everything but the loads of the last kAhead-1 steps has landed: activations and     */      \
-                /* weights of step k+1. The next quad's scales were asked for at the head of step 0,    */      \
-                /* behind the loads of the step before: with more than one step in flight they lie      */      \
-                /* inside that window, and step 0 leaves them in flight too.                            */      \
-                wait_loads_but<(kAhead - 1) * kPerStep + ((b) == 0 && kAhead > 2 ? 4 + TT : 0)>();              \
-                lds_barrier(); /* with the wait for this group's fragment */                                   \
-                read_fragment(flo, fhi, aring_at + ar1 * TT * 2048);                                           \
-                read_weights(af[((b) + 1) & 1], wr1);                                                          \
+                if (NEXT) {                                                                                    \
+                    /* Everything but the ALLOW youngest loads has landed: activations and weights of   */      \
+                    /* step k+1 are older than those.                                                   */      \
+                    wait_loads_but<(ALLOW)>();                                                                 \
+                    lds_barrier(); /* with the wait for this group's fragment */                               \
+                    read_fragment(flo, fhi, aring_at + ar1 * TT * 2048);                                       \
+                    read_weights(af[((b) + 1) & 1], wr1);                                                      \
+                } else {                                                                                       \
+                    wait_lds_but<0>(); /* the chunk's last step: nothing to fetch, nobody to wait for */      \
+                }                                                                                              \
             } else {                                                                                           \
                 wait_lds_but<0>();                                                                             \
             }                                                                                                  \
@@ -266,7 +271,7 @@ __device__ __forceinline__ void gemm_chunk_lds(v4f (&acc)[4][TT], const uint8_t*
             __builtin_amdgcn_sched_barrier(0);                                                                 \
             mfma_acc<(b)>(acc[2][tt], af[(b) & 1][2], bv, SW[2], SA[tt]);                                       \
             __builtin_amdgcn_sched_barrier(0);                                                                 \
-            if (tt + 1 < TT) {                                                                                 \
+            if (STAGE && tt + 1 < TT) {                                                                        \
                 _Pragma("unroll") for (int item = 0; item < kPerStep; ++item)                                  \
                     if (item * TT / kPerStep == tt) stage_item(item, ahead, ar2, wr);                          \
             }                                                                                                  \
@@ -279,30 +284,58 @@ __device__ __forceinline__ void gemm_chunk_lds(v4f (&acc)[4][TT], const uint8_t*
         wr = wr1;                                                                                              \
         ar = ar1;                                                                                              \
     }
-    // A quad: fetch the next quad's scales into the other set, then four k-steps on this set.
+    // A quad: fetch the next quad's scales into the other set, then four k-steps on this set. A step leaves
+    // the loads of the kAhead-1 steps behind the next one in flight; the next quad's scales were asked for at
+    // the head of step 0, behind the loads of the step before, so with more than one step in flight they lie
+    // inside that window and step 0 leaves them in flight too.
+#define M26G_ALLOW(b) ((kAhead - 1) * kPerStep + ((b) == 0 && kAhead > 2 ? 4 + TT : 0))
 #define M26G_QUAD(SW, SA, NW, NA)                                                                              \
     {                                                                                                          \
-        load_scales(NW, NA, q + 1 < quads ? q + 1 : q);                                                        \
+        load_scales(NW, NA, q + 1);                                                                            \
         __builtin_amdgcn_sched_barrier(0);                                                                     \
-        M26G_KSTEP(0, SW, SA)                                                                                  \
-        M26G_KSTEP(1, SW, SA)                                                                                  \
-        M26G_KSTEP(2, SW, SA)                                                                                  \
-        M26G_KSTEP(3, SW, SA)                                                                                  \
+        M26G_KSTEP(0, SW, SA, 1, M26G_ALLOW(0), 1)                                                             \
+        M26G_KSTEP(1, SW, SA, 1, M26G_ALLOW(1), 1)                                                             \
+        M26G_KSTEP(2, SW, SA, 1, M26G_ALLOW(2), 1)                                                             \
+        M26G_KSTEP(3, SW, SA, 1, M26G_ALLOW(3), 1)                                                             \
         /* The compiler may put anything behind a quad, a copy of an accumulator included (it hands them to */ \
         /* the code after the loop in other registers when it likes), and it does not know that the last  */ \
         /* MFMA's result is eight passes away: sixteen wait states cover that with room to spare.         */ \
         asm volatile("s_nop 15" ::: "memory");                                                                \
         ++q;                                                                                                   \
     }
-#pragma unroll 1
-    while (q + 1 < quads) {
-        M26G_QUAD(sw0, sa0, sw1, sa1)
-        M26G_QUAD(sw1, sa1, sw0, sa0)
+    // The chunk's last quad stages only the steps that exist (step j stages step j + kAhead of the quad),
+    // leaves in flight only what is younger than the step after it, and its last step fetches nothing
+    // and meets nobody: no load is issued for a step past the end.
+#define M26G_TAIL_STAGE(j) ((j) + kAhead <= 3)
+#define M26G_TAIL_ALLOW(j) (((kAhead - 1) < (2 - (j)) ? (kAhead - 1) : (2 - (j))) * kPerStep)
+#define M26G_TAIL(SW, SA)                                                                                      \
+    {                                                                                                          \
+        M26G_KSTEP(0, SW, SA, M26G_TAIL_STAGE(0), M26G_TAIL_ALLOW(0), 1)                                       \
+        M26G_KSTEP(1, SW, SA, M26G_TAIL_STAGE(1), M26G_TAIL_ALLOW(1), 1)                                       \
+        M26G_KSTEP(2, SW, SA, M26G_TAIL_STAGE(2), M26G_TAIL_ALLOW(2), 1)                                       \
+        M26G_KSTEP(3, SW, SA, 0, 0, 0)                                                                         \
+        asm volatile("s_nop 15" ::: "memory");                                                                \
+        ++q;                                                                                                   \
     }
-    if (q < quads) M26G_QUAD(sw0, sa0, sw1, sa1)  // odd count: an even number of quads ends on set 0
+    if constexpr (ONE) {
+        M26G_TAIL(sw0, sa0)
+    } else {
+        const int whole = quads - 1;  // quads that have a quad behind them: an odd number
+#pragma unroll 1
+        while (q + 1 < whole) {
+            M26G_QUAD(sw0, sa0, sw1, sa1)
+            M26G_QUAD(sw1, sa1, sw0, sa0)
+        }
+        M26G_QUAD(sw0, sa0, sw1, sa1)
+        M26G_TAIL(sw1, sa1)
+    }
+#undef M26G_TAIL
+#undef M26G_TAIL_ALLOW
+#undef M26G_TAIL_STAGE
+#undef M26G_ALLOW
 #undef M26G_QUAD
 #undef M26G_KSTEP
-    wait_loads_but<0>();  // the re-staged tail loads must land before the LDS is reused or the wave ends
+    wait_loads_but<0>();  // nothing is left in flight by now; the LDS is about to be reused
     wait_lds_but<0>();
     // The last fetches of scales, fragment and weights feed no MFMA. To the compiler such a register is
     // free the moment the load has issued, and whatever it puts there next is overwritten when the
@@ -350,7 +383,7 @@ __device__ __forceinline__ void fc1_tile_body(const Fc1Args& a, const Chunk ch, 
     for (int t = 0; t < 4; ++t)
 #pragma unroll
         for (int tt = 0; tt < TT; ++tt) acc[t][tt] = v4f{0.f, 0.f, 0.f, 0.f};
-    gemm_chunk_lds<S, TT>(acc, wp, sp, sx, int(kHidden / 128), row, wv, lane, lds);
+    gemm_chunk_lds<S, TT, false>(acc, wp, sp, sx, int(kHidden / 128), row, wv, lane, lds);
     const uint32_t lane2 = after_loop(lane), r2 = lane2 & 15;
     const uint32_t verdict = a.rowbad[c * 16 + r2], bad = verdict & 1u;
     // The accumulators leave the accumulation registers through LDS, sixteen tiles at a time: whole-tile
@@ -388,7 +421,7 @@ __device__ __forceinline__ void fc1_tile_body(const Fc1Args& a, const Chunk ch, 
 // FC2 for chunk c by one workgroup: 256 output columns x 16*TT rows; the wave owns block ob.
 // `verdict` is rowbad[c][lane % 16] (bit 8+t: tile t holds a token in this row), fetched by the caller beside
 // the chunk record.
-template <class S, int TT>
+template <class S, int TT, bool ONE>
 __device__ __forceinline__ void fc2_tile_body(const Fc2Args& a, const Chunk ch, uint32_t c, uint32_t ob, uint32_t wv,
                                               uint32_t lane, uint8_t* lds, const uint32_t verdict) {
     constexpr int kMine = staged_tiles<S, TT>();
@@ -412,7 +445,7 @@ __device__ __forceinline__ void fc2_tile_body(const Fc2Args& a, const Chunk ch, 
     for (int t = 0; t < 4; ++t)
 #pragma unroll
         for (int tt = 0; tt < TT; ++tt) acc[t][tt] = v4f{0.f, 0.f, 0.f, 0.f};
-    gemm_chunk_lds<S, TT>(acc, wp, sp, sx, int(ksteps), row, wv, lane, lds);
+    gemm_chunk_lds<S, TT, ONE>(acc, wp, sp, sx, int(ksteps), row, wv, lane, lds);
     const uint32_t lane2 = after_loop(lane);
     // A lane holds four consecutive output columns of one token per tile, so a store straight from the
     // accumulators touches sixteen token rows with 64 bytes each. One trip through the wave's own, now
@@ -498,8 +531,9 @@ __global__ void __launch_bounds__(S::kThreads, 8 / S::kWaves) fc1_tile_kernel(Fc
     else fc1_tile_body<S, 8>(a, ch, c, cb, wv, lane, lds, token8);
 }
 
-// One workgroup per (chunk, 64 * kWaves output columns).
-template <class S>
+// One workgroup per (chunk, 64 * kWaves output columns). ONE: the layer holds one rank's share (I = 512, a single
+// quad of k-steps); otherwise I = 2048.
+template <class S, bool ONE>
 __global__ void __launch_bounds__(S::kThreads, 8 / S::kWaves) fc2_tile_kernel(Fc2Args a) {
     extern __shared__ __align__(16) uint8_t lds[];
     uint32_t* meta = a.plan.meta;
@@ -517,8 +551,8 @@ __global__ void __launch_bounds__(S::kThreads, 8 / S::kWaves) fc2_tile_kernel(Fc
     }
     if (ch.groups == 1) fc2_body<1>(a, ch, ob, lane);
     else if (ch.groups == 2) fc2_body<2>(a, ch, ob, lane);
-    else if (ch.groups <= 4) fc2_tile_body<S, 4>(a, ch, c, ob, wv, lane, lds, verdict);
-    else fc2_tile_body<S, 8>(a, ch, c, ob, wv, lane, lds, verdict);
+    else if (ch.groups <= 4) fc2_tile_body<S, 4, ONE>(a, ch, c, ob, wv, lane, lds, verdict);
+    else fc2_tile_body<S, 8, ONE>(a, ch, c, ob, wv, lane, lds, verdict);
 }
 
 }  // namespace m26g

@@ -105,4 +105,4 @@ def test_checker_follows_the_control_flow():
 
 def test_built_tile_kernels_pass():
     seen = codegen_check.run()
-    assert len(seen) == 2 and all(n >= 100 for n in seen.values())
+    assert len(seen) == 3 and all(n >= 100 for n in seen.values())
