@@ -69,11 +69,11 @@ uint32_t m26s_b1_layer_intermediate(const m26s_b1_layer* layer);
 /* The prepared pool of a layer, for persisting it or checking it: 256 images of *image_bytes each
  * (3,342,336 for one rank's share, four times that for a full layer) in expert-id order, device
  * memory owned by the layer. *layout_tag names the byte order (the counterpart of the reference's
- * prepared tag, crates/mimo26-expert/kernels/b1/prepared.cuh:16-31): M26S_B1_LAYOUT_G950_V1 is
+ * prepared tag, crates/mimo26-expert/kernels/b1/prepared.cuh:16-31): M26S_B1_LAYOUT_G950_V2 is
  * the operand order of gfx950's v_mfma_scale_f32_16x16x128_f8f6f4 this library writes; a persisted
  * pool carrying any other tag must be prepared again from the canonical images. Returns 0, or 1
  * for a null argument. */
-#define M26S_B1_LAYOUT_G950_V1 0x47393501u /* "G95" 0x01 */
+#define M26S_B1_LAYOUT_G950_V2 0x47393502u /* "G95" 0x02 */
 int m26s_b1_layer_view(const m26s_b1_layer* layer, const uint8_t** prepared_dev, uint64_t* image_bytes,
                        uint32_t* layout_tag);
 

@@ -299,7 +299,7 @@ template <int NT>
 void launch_direct(const m26s_b1_layer* L, const Launch& k, const Fc1Args& f1, const Fc2Args& f2) {
     fc1_kernel<NT><<<dim3(L->lay.inter / 128, k.ws.chunk_cap), 256, 0, k.stream>>>(f1);
     mark(k.fc1_done, k.stream);
-    fc2_kernel<NT><<<dim3(16 / kFc2Blocks, k.ws.chunk_cap), 256, 0, k.stream>>>(f2);
+    fc2_kernel<NT><<<dim3(16, k.ws.chunk_cap), 256, 0, k.stream>>>(f2);
     mark(k.fc2_done, k.stream);
 }
 // Prefill-size calls: workgroups that share each chunk's activation tiles through LDS, two per compute unit.
@@ -469,7 +469,7 @@ int m26s_b1_layer_view(const m26s_b1_layer* L, const uint8_t** prepared_dev, uin
     if (!L || !prepared_dev || !image_bytes || !layout_tag) return 1;
     *prepared_dev = L->prepared;
     *image_bytes = L->lay.bytes();
-    *layout_tag = M26S_B1_LAYOUT_G950_V1;
+    *layout_tag = M26S_B1_LAYOUT_G950_V2;
     return 0;
 }
 

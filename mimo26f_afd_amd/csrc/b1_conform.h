@@ -55,7 +55,7 @@ __device__ __forceinline__ float activation_value(uint32_t code, uint32_t s) {
 struct WeightCell { uint64_t payload, scale; };
 __device__ __forceinline__ WeightCell weight_cell(uint32_t block, uint32_t t, uint32_t row16, uint32_t kb, uint32_t ksteps) {
     const uint32_t ks = kb >> 2, lane = 16 * (kb & 3u) + row16;
-    return WeightCell{((uint64_t(block) * ksteps + ks) * 4 + t) * 1024 + lane * 16,
+    return WeightCell{block_payload(block, ksteps) + uint64_t(ks) * kStepBytes + t * 1024 + lane * 16,
                       ((uint64_t(block) * (ksteps / 4) + (ks >> 2)) * 4 + t) * 256 + lane * 4 + (ks & 3u)};
 }
 

@@ -48,7 +48,7 @@ __global__ void __launch_bounds__(256) prepare_kernel(Canonical c, uint8_t* __re
     const uint32_t stride = gridDim.x * blockDim.x, first = blockIdx.x * blockDim.x + threadIdx.x;
     bool odd = false;
     for (uint32_t cell = first; cell < I * 256; cell += stride) {  // w13 payload
-        const uint32_t lane = cell & 63, t = (cell >> 6) & 3, ks = (cell >> 8) & 31, cb = cell >> 13;
+        const uint32_t lane = cell & 63, t = (cell >> 6) & 3, ks = (cell >> 11) & 31, cb = (cell >> 16) * kSetBlocks + ((cell >> 8) & 7);
         const uint32_t n = cb * 32 + (t & 1) * 16 + (lane & 15), g = lane >> 4;
         const uint8_t* src = c.pool[n / kRankI] + img + (t < 2 ? kGatePayload : kUpPayload) +
                              uint64_t(n % kRankI) * 2048 + ks * 64 + g * 16;
@@ -68,7 +68,8 @@ __global__ void __launch_bounds__(256) prepare_kernel(Canonical c, uint8_t* __re
     }
     const uint32_t ksteps = I / 128, quads = I / 512;
     for (uint32_t cell = first; cell < I * 128; cell += stride) {  // w2 payload
-        const uint32_t lane = cell & 63, t = (cell >> 6) & 3, ks = (cell >> 8) % ksteps, ob = (cell >> 8) / ksteps;
+        const uint32_t lane = cell & 63, t = (cell >> 6) & 3, ks = (cell >> 11) % ksteps;
+        const uint32_t ob = (cell >> 11) / ksteps * kSetBlocks + ((cell >> 8) & 7);
         const uint32_t n = ob * 64 + t * 16 + (lane & 15), kb = 4 * ks + (lane >> 4);
         const uint8_t* src = c.pool[kb / 16] + img + kDownPayload + uint64_t(n) * 256 + (kb % 16) * 16;
         *reinterpret_cast<uint4*>(dst + lay.w2() + uint64_t(cell) * 16) = *reinterpret_cast<const uint4*>(src);
@@ -567,9 +568,7 @@ __global__ void __launch_bounds__(256) quantize_kernel(const float* __restrict__
 //
 // One wave owns four 16-row weight tiles (SrcA, FP4, streamed once, fully coalesced 1 KB per
 // tile per k-step) and TT 16-row activation tiles (SrcB, FP8, row-major rows gathered by
-// pointer). A k-step is K = 128. Loads for step k+1 are issued before the MFMAs of step k.
-// The walk over K starts at quad `first` and wraps, so waves that stream neighbouring weight
-// blocks do not sit on the same addresses modulo the block size at the same time.
+// pointer). A k-step is K = 128; a block's next k-step lies kStepBytes further on.
 // ---------------------------------------------------------------------------------------------
 // Weight fragments of one k-step (four tiles) and the activation fragments of one k-step.
 struct WeightStep { v4i a[4]; };
@@ -581,7 +580,7 @@ struct ActStep {
 
 __device__ __forceinline__ void load_weights(WeightStep& o, const uint8_t* __restrict__ wp, int ks) {
 #pragma unroll
-    for (int t = 0; t < 4; ++t) o.a[t] = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(wp + size_t(ks) * 4096 + t * 1024));
+    for (int t = 0; t < 4; ++t) o.a[t] = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(wp + size_t(ks) * kStepBytes + t * 1024));
 }
 template <int TT>
 __device__ __forceinline__ void load_acts(ActStep<TT>& o, int ks, const uint8_t* const (&xrow)[TT],
@@ -613,27 +612,18 @@ __device__ __forceinline__ void mfma_step(v4f (&acc)[4][TT], const WeightStep& w
 
 // wp / sp already include the lane offset (lane*16, lane*4). ksteps is a multiple of 4.
 //
-// This is the schedule of the HBM-bound sizes, so what counts is bytes in flight: the weight stream
-// (4 KB per wave and k-step, each byte used once) runs three k-steps ahead of the MFMAs in a ring of
-// four register sets, about 12 KB per wave and 36 KB per SIMD at three waves, which is what 7 TB/s
-// times the memory latency asks for. Activation rows come from L2 and run one k-step ahead; the
-// weight scale dwords of the next quad of k-steps are fetched a quad ahead. Past the end the last
-// k-step is fetched again rather than branching.
-// `blocks` consecutive weight blocks (their fragments and scale dwords lie back to back) against the
-// same activation rows, one after the other: the weight stream does not restart between them, the
-// accumulators are handed to `done(b)` after block b and cleared. One block is the plain case.
-template <int TT, class Done>
-__device__ __forceinline__ void gemm_blocks(v4f (&acc)[4][TT], const uint8_t* __restrict__ wp,
-                                            const uint8_t* __restrict__ sp, int ksteps, int blocks,
-                                            const uint8_t* const (&xrow)[TT], const uint8_t* const (&xsrow)[TT],
-                                            uint32_t lane, uint32_t& bad, Done done) {
+// This is the schedule of the HBM-bound sizes: the weight stream (4 KB per wave and k-step, each byte used
+// once) is asked for three k-steps ahead of the MFMAs in a ring of four register sets; activation rows come
+// from L2 and run one k-step ahead; the weight scale dwords of the next quad of k-steps are fetched a quad
+// ahead. Past the end the last k-step is fetched again rather than branching.
+template <int TT>
+__device__ __forceinline__ void gemm_chunk(v4f (&acc)[4][TT], const uint8_t* __restrict__ wp,
+                                           const uint8_t* __restrict__ sp, int ksteps,
+                                           const uint8_t* const (&xrow)[TT], const uint8_t* const (&xsrow)[TT],
+                                           uint32_t lane, uint32_t& bad) {
     const uint32_t shift = 8 * (lane >> 4);
-    const int quads = ksteps / 4, last = blocks * ksteps - 1, last_quad = blocks * quads - 1;
-    auto weights_at = [&](int g) { return g < last ? g : last; };
-    auto acts_at = [&](int local, int g) {  // the rows start over with every block; `local` counts inside block b
-        local -= g > last ? g - last : 0;
-        return local >= ksteps ? local - ksteps : local;
-    };
+    const int quads = ksteps / 4, last = ksteps - 1;
+    auto upto = [&](int g) { return g < last ? g : last; };
     WeightStep w[4];
     ActStep<TT> x[2];
     uint32_t sw[4], swn[4];
@@ -643,39 +633,29 @@ __device__ __forceinline__ void gemm_blocks(v4f (&acc)[4][TT], const uint8_t* __
     load_acts<TT>(x[0], 0, xrow, xsrow);
 #pragma unroll
     for (int t = 0; t < 4; ++t) sw[t] = *reinterpret_cast<const uint32_t*>(sp + t * 256);
-    for (int b = 0; b < blocks; ++b) {
 #pragma unroll
-        for (int t = 0; t < 4; ++t)
+    for (int t = 0; t < 4; ++t)
 #pragma unroll
-            for (int tt = 0; tt < TT; ++tt) acc[t][tt] = v4f{0.f, 0.f, 0.f, 0.f};
-        for (int q = 0; q < quads; ++q) {
-            const int g = b * ksteps + 4 * q, gq = b * quads + q, qn = gq < last_quad ? gq + 1 : last_quad;
+        for (int tt = 0; tt < TT; ++tt) acc[t][tt] = v4f{0.f, 0.f, 0.f, 0.f};
+    for (int q = 0; q < quads; ++q) {
+        const int g = 4 * q, qn = q + 1 < quads ? q + 1 : q;
 #pragma unroll
-            for (int t = 0; t < 4; ++t) swn[t] = *reinterpret_cast<const uint32_t*>(sp + size_t(qn) * 1024 + t * 256);
-            load_weights(w[3], wp, g + 3);
-            load_acts<TT>(x[1], acts_at(4 * q + 1, g + 1), xrow, xsrow);
-            mfma_step<TT, 0>(acc, w[0], x[0], sw, shift, bad);
-            load_weights(w[0], wp, weights_at(g + 4));
-            load_acts<TT>(x[0], acts_at(4 * q + 2, g + 2), xrow, xsrow);
-            mfma_step<TT, 1>(acc, w[1], x[1], sw, shift, bad);
-            load_weights(w[1], wp, weights_at(g + 5));
-            load_acts<TT>(x[1], acts_at(4 * q + 3, g + 3), xrow, xsrow);
-            mfma_step<TT, 2>(acc, w[2], x[0], sw, shift, bad);
-            load_weights(w[2], wp, weights_at(g + 6));
-            load_acts<TT>(x[0], acts_at(4 * q + 4, g + 4), xrow, xsrow);
-            mfma_step<TT, 3>(acc, w[3], x[1], sw, shift, bad);
+        for (int t = 0; t < 4; ++t) swn[t] = *reinterpret_cast<const uint32_t*>(sp + size_t(qn) * 1024 + t * 256);
+        load_weights(w[3], wp, g + 3);
+        load_acts<TT>(x[1], g + 1, xrow, xsrow);
+        mfma_step<TT, 0>(acc, w[0], x[0], sw, shift, bad);
+        load_weights(w[0], wp, upto(g + 4));
+        load_acts<TT>(x[0], g + 2, xrow, xsrow);
+        mfma_step<TT, 1>(acc, w[1], x[1], sw, shift, bad);
+        load_weights(w[1], wp, upto(g + 5));
+        load_acts<TT>(x[1], g + 3, xrow, xsrow);
+        mfma_step<TT, 2>(acc, w[2], x[0], sw, shift, bad);
+        load_weights(w[2], wp, upto(g + 6));
+        load_acts<TT>(x[0], upto(g + 4), xrow, xsrow);
+        mfma_step<TT, 3>(acc, w[3], x[1], sw, shift, bad);
 #pragma unroll
-            for (int t = 0; t < 4; ++t) sw[t] = swn[t];
-        }
-        done(b);
+        for (int t = 0; t < 4; ++t) sw[t] = swn[t];
     }
-}
-template <int TT>
-__device__ __forceinline__ void gemm_chunk(v4f (&acc)[4][TT], const uint8_t* __restrict__ wp,
-                                           const uint8_t* __restrict__ sp, int ksteps,
-                                           const uint8_t* const (&xrow)[TT], const uint8_t* const (&xsrow)[TT],
-                                           uint32_t lane, uint32_t& bad) {
-    gemm_blocks<TT>(acc, wp, sp, ksteps, 1, xrow, xsrow, lane, bad, [](int) {});
 }
 
 // e^t for t <= 0 in binary32 on the hardware 2^x: the product t * log2(e) is formed as a rounded head and
@@ -832,7 +812,7 @@ __device__ __forceinline__ void fc1_body(const Fc1Args& a, const Chunk ch, uint3
         xsrow[tt] = live[tt] ? a.xs + size_t(row) * a.xs_pitch : a.unit_scales;
     }
     const uint8_t* img = a.prepared + uint64_t(expert) * a.lay.bytes();
-    const uint8_t* wp = img + a.lay.w13() + uint64_t(cb) * (32 * 4096) + lane * 16;
+    const uint8_t* wp = img + a.lay.w13() + block_payload(cb, 32) + lane * 16;
     const uint8_t* sp = img + a.lay.s13() + uint64_t(cb) * (8 * 1024) + lane * 4;
     v4f acc[4][TT];
 #pragma unroll
@@ -912,10 +892,9 @@ __device__ __forceinline__ void fc2_finish(const Fc2Args& a, uint32_t ob, uint32
     if (lost) atomicOr(&a.plan.meta[kFc2Fault], 5u);
 }
 
-// One wave's share of FC2 for a chunk of TT groups: 64 output columns x 16*TT rows per block, `blocks`
-// neighbouring blocks from `ob` on in one uninterrupted weight stream.
+// One wave's share of FC2 for a chunk of TT groups: 64 output columns x 16*TT rows.
 template <int TT>
-__device__ __forceinline__ void fc2_body(const Fc2Args& a, const Chunk ch, uint32_t ob, uint32_t lane, uint32_t blocks = 1) {
+__device__ __forceinline__ void fc2_body(const Fc2Args& a, const Chunk ch, uint32_t ob, uint32_t lane) {
     const uint32_t r = lane & 15, g = lane >> 4, I = a.lay.inter;
     const Group* grp = a.plan.groups + ch.first_group;
     const int32_t expert = ch.expert;
@@ -932,20 +911,18 @@ __device__ __forceinline__ void fc2_body(const Fc2Args& a, const Chunk ch, uint3
     }
     const uint32_t ksteps = I / 128;
     const uint8_t* img = a.prepared + uint64_t(expert) * a.lay.bytes();
-    const uint8_t* wp = img + a.lay.w2() + uint64_t(ob) * ksteps * 4096 + lane * 16;
+    const uint8_t* wp = img + a.lay.w2() + block_payload(ob, ksteps) + lane * 16;
     const uint8_t* sp = img + a.lay.s2() + uint64_t(ob) * (ksteps / 4) * 1024 + lane * 4;
     v4f acc[4][TT];
     uint32_t bad = 0;
-    gemm_blocks<TT>(acc, wp, sp, int(ksteps), int(blocks), xrow, xsrow, lane, bad,
-                    [&](int b) { fc2_finish<TT>(a, ob + uint32_t(b), lane, acc, route); });
+    gemm_chunk<TT>(acc, wp, sp, int(ksteps), xrow, xsrow, lane, bad);
+    fc2_finish<TT>(a, ob, lane, acc, route);
 }
 
 // Stage 4a: down grouped GEMM on the requantised intermediate; rows go back to y[original route].
-// grid (16 / kFc2Blocks, chunk capacity), 256 threads; each wave owns kFc2Blocks x 64 output columns, one
-// block after the other in one weight stream. FC2's stream per block is half as long as FC1's (K = I against
-// K = H), but two blocks per wave halve the workgroups, and at 128 tokens the longer tail of the launch costs
-// more than the longer streams save (172 against 154 us): one block it is.
-constexpr uint32_t kFc2Blocks = 1;
+// grid (16, chunk capacity), 256 threads; each wave owns 64 output columns. (Two neighbouring blocks per wave
+// in one stream halve the workgroups, and at 128 tokens the longer tail of the launch cost more than the longer
+// streams saved, 172 against 154 us.)
 template <int NT>
 __global__ void __launch_bounds__(256) fc2_kernel(Fc2Args a) {
     uint32_t* meta = a.plan.meta;
@@ -953,16 +930,16 @@ __global__ void __launch_bounds__(256) fc2_kernel(Fc2Args a) {
     const ItemHead head = load_item_head(a.plan.chunks + c, meta);
     const Chunk ch = head.ch;
     if (head.meta[kPlanFault] || head.meta[kFc1Fault] || head.meta[kQuantFault] || c >= head.meta[kChunkCount]) return;
-    const uint32_t lane = threadIdx.x & 63, ob = (blockIdx.x * 4 + (threadIdx.x >> 6)) * kFc2Blocks;
+    const uint32_t lane = threadIdx.x & 63, ob = blockIdx.x * 4 + (threadIdx.x >> 6);
     const int32_t expert = ch.expert;
     if (expert < 0 || expert >= int32_t(kExperts) || ch.groups < 1 || ch.groups > NT) {
         if (lane == 0) atomicOr(&meta[kFc2Fault], 2u);
         return;
     }
-    if (NT == 1 || ch.groups == 1) fc2_body<1>(a, ch, ob, lane, kFc2Blocks);
-    else if (NT == 2 || ch.groups == 2) fc2_body<2>(a, ch, ob, lane, kFc2Blocks);
-    else if (NT >= 4 && ch.groups <= 4) fc2_body<(NT >= 4 ? 4 : 1)>(a, ch, ob, lane, kFc2Blocks);
-    else fc2_body<(NT >= 8 ? 8 : 1)>(a, ch, ob, lane, kFc2Blocks);
+    if (NT == 1 || ch.groups == 1) fc2_body<1>(a, ch, ob, lane);
+    else if (NT == 2 || ch.groups == 2) fc2_body<2>(a, ch, ob, lane);
+    else if (NT >= 4 && ch.groups <= 4) fc2_body<(NT >= 4 ? 4 : 1)>(a, ch, ob, lane);
+    else fc2_body<(NT >= 8 ? 8 : 1)>(a, ch, ob, lane);
 }
 
 // Stage 4b: router-weighted combine. Per (token, column): v = 0; for slot 0..7:

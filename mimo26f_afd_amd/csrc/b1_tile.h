@@ -173,7 +173,7 @@ __device__ __forceinline__ void gemm_chunk_lds(v4f (&acc)[4][TT], const uint8_t*
             load_row_to_lds(row[m] + ks * 128 + half * 64, aring + (astage * TT * 2 + cell) * 1024);
         } else {
             const int t = item - kCells;
-            load_row_to_lds(wp + size_t(ks) * 4096 + t * 1024, wring + wstage * 4096 + t * 1024);
+            load_row_to_lds(wp + size_t(ks) * kStepBytes + t * 1024, wring + wstage * 4096 + t * 1024);
         }
     };
     auto stage_all = [&](int ks, uint32_t astage, uint32_t wstage) {
@@ -375,7 +375,7 @@ __device__ __forceinline__ void fc1_tile_body(const Fc1Args& a, const Chunk ch, 
 #pragma unroll
     for (int m = 0; m < kMine; ++m) row[m] = (token[m] >= 0 ? a.x + size_t(token[m]) * a.x_pitch : a.zero_row) + g * 16;
     const uint8_t* img = a.prepared + uint64_t(expert) * a.lay.bytes();
-    const uint8_t* wp = img + a.lay.w13() + uint64_t(cb) * (32 * 4096) + lane * 16;
+    const uint8_t* wp = img + a.lay.w13() + block_payload(cb, 32) + lane * 16;
     const uint8_t* sp = img + a.lay.s13() + uint64_t(cb) * (8 * 1024) + lane * 4;
     const uint8_t* sx = a.xg + size_t(c) * gathered_scale_bytes(kHidden) + lane * 4;
     v4f acc[4][TT];
@@ -437,7 +437,7 @@ __device__ __forceinline__ void fc2_tile_body(const Fc2Args& a, const Chunk ch, 
     }
     const uint32_t ksteps = I / 128;
     const uint8_t* img = a.prepared + uint64_t(expert) * a.lay.bytes();
-    const uint8_t* wp = img + a.lay.w2() + uint64_t(ob) * ksteps * 4096 + lane * 16;
+    const uint8_t* wp = img + a.lay.w2() + block_payload(ob, ksteps) + lane * 16;
     const uint8_t* sp = img + a.lay.s2() + uint64_t(ob) * (ksteps / 4) * 1024 + lane * 4;
     const uint8_t* sx = a.dg + size_t(c) * gathered_scale_bytes(I) + lane * 4;
     v4f acc[4][TT];

@@ -11,7 +11,7 @@ sha, a drifted geometry or layout row, a slice of the wrong size or hash refuses
 
 `load_layer` is this build's end of it: the verified slices of one layer go to the GPU (one rank's
 256 images, or all four ranks for a full-intermediate layer) and are permuted once into the gfx950
-operand order by the library (layout tag M26S_B1_LAYOUT_G950_V1).
+operand order by the library (layout tag M26S_B1_LAYOUT_G950_V2).
 """
 from __future__ import annotations
 
@@ -35,7 +35,7 @@ GEOMETRY = {"hidden": HIDDEN, "intermediate": INTERMEDIATE, "experts_per_layer":
 LAYOUT = (("gate_proj", "payload", 0, 1048576), ("gate_proj", "scales", 1048576, 65536),
           ("up_proj", "payload", 1114112, 1048576), ("up_proj", "scales", 2162688, 65536),
           ("down_proj", "payload", 2228224, 1048576), ("down_proj", "scales", 3276800, 65536))
-LAYOUT_TAG_G950_V1 = 0x47393501
+LAYOUT_TAG_G950_V2 = 0x47393502
 _PROJ = (("gate_proj", 2048, 4096), ("up_proj", 2048, 4096), ("down_proj", 4096, 2048))  # name, out rows, in cols
 
 
@@ -336,6 +336,6 @@ def load_layer(directory: str, layer: int, rank: int | None = 0) -> b1.Layer:
     finally:
         for p in pools:
             p.free()
-    if made.prepared_view()[2] != LAYOUT_TAG_G950_V1:
+    if made.prepared_view()[2] != LAYOUT_TAG_G950_V2:
         raise IngestError("BadLayout", "the library prepared a layout this loader does not know")
     return made

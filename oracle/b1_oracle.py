@@ -186,9 +186,11 @@ def prepared_g950(images) -> np.ndarray:
     (crates/mimo26-expert/tests/b1/host.cpp:30-67). Raises if the map is not a bijection.
 
     Destination, I = 512 * len(images) intermediate columns, lane = 16 * (k-block % 4) + row % 16:
-      gate/up payload  [I/32][32 k-steps][4 tiles][64 lanes][16 B], tile = (row % 32) // 16 + (2 for up)
+      gate/up payload  [I/256][32 k-steps][8 blocks][4 tiles][64 lanes][16 B], block = row // 32 (its set of
+                       eight = block // 8, place in the set = block % 8), tile = (row % 32) // 16 + (2 for up)
       gate/up scales   [I/32][8][4 tiles][64 lanes][4 B], byte = k-step % 4 of quad k-step // 4
-      down payload     [64][I/128 k-steps][4 tiles][64 lanes][16 B], tile = (row % 64) // 16
+      down payload     [8][I/128 k-steps][8 blocks][4 tiles][64 lanes][16 B], block = row // 64,
+                       tile = (row % 64) // 16
       down scales      [64][I/512][4 tiles][64 lanes][4 B]
     with k-block = k // 32 and k-step = k-block // 4; the down projection's K runs over the ranks."""
     ranks = len(images)
@@ -213,7 +215,7 @@ def prepared_g950(images) -> np.ndarray:
             kb, within = b // 16, b % 16
             lane = 16 * (kb % 4) + n % 16
             tile = (n % 32) // 16 + 2 * up
-            put(w13 + ((((n // 32) * 32 + kb // 4) * 4 + tile) * 64 + lane) * 16 + within, img[pay:pay + 512 * 2048].reshape(512, 2048))
+            put(w13 + ((((((n // 256) * 32 + kb // 4) * 8 + (n // 32) % 8) * 4 + tile) * 64 + lane) * 16 + within), img[pay:pay + 512 * 2048].reshape(512, 2048))
             kb = np.arange(128)[None, :]
             lane = 16 * (kb % 4) + n % 16
             step = kb // 4
@@ -223,7 +225,7 @@ def prepared_g950(images) -> np.ndarray:
         kb, within = r * 16 + b // 16, b % 16
         lane = 16 * (kb % 4) + n % 16
         tile = (n % 64) // 16
-        put(w2 + ((((n // 64) * (inter // 128) + kb // 4) * 4 + tile) * 64 + lane) * 16 + within, img[2228224:2228224 + 4096 * 256].reshape(4096, 256))
+        put(w2 + ((((((n // 512) * (inter // 128) + kb // 4) * 8 + (n // 64) % 8) * 4 + tile) * 64 + lane) * 16 + within), img[2228224:2228224 + 4096 * 256].reshape(4096, 256))
         kb = r * 16 + np.arange(16)[None, :]
         lane = 16 * (kb % 4) + n % 16
         step = kb // 4

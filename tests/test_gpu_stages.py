@@ -183,7 +183,7 @@ def test_prepared_pool_is_the_forward_map_of_the_canonical_images(ranks):
     layer = DeviceLayer(pools).layer
     assert layer.intermediate == 512 * ranks and not layer.all_scales_normal()
     ptr, image_bytes, tag = layer.prepared_view()
-    assert image_bytes == ranks * synth.IMAGE_BYTES and tag == 0x47393501
+    assert image_bytes == ranks * synth.IMAGE_BYTES and tag == 0x47393502
     for e in experts + (7,):
         got = np.empty(image_bytes, np.uint8)
         assert b1.load().m26s_b1_copy_to_host(got.ctypes.data, ptr + e * image_bytes, image_bytes) == 0

@@ -156,7 +156,7 @@ def test_layer_from_slice_files_equals_layer_from_pool(tmp_path):
     make_dir(tmp_path, images)
     layer = G.load_layer(str(tmp_path), 3, rank=0)
     ptr, image_bytes, tag = layer.prepared_view()
-    assert tag == G.LAYOUT_TAG_G950_V1 and image_bytes == synth.IMAGE_BYTES and layer.all_scales_normal()
+    assert tag == G.LAYOUT_TAG_G950_V2 and image_bytes == synth.IMAGE_BYTES and layer.all_scales_normal()
     e = int(wl.ids[0, 0])
     got = np.empty(image_bytes, np.uint8)
     assert b1.load().m26s_b1_copy_to_host(got.ctypes.data, ptr + e * image_bytes, image_bytes) == 0
