@@ -23,6 +23,7 @@ sys.path.insert(0, os.path.join(ROOT, "oracle"))
 
 HBM_PEAK_GBS = 8000.0           # MI355X HBM3E, published
 MFMA_FP8_PEAK_TFLOPS = 5000.0   # dense FP8 (an FP8 x FP4 block-scaled MFMA issues at the FP8 rate)
+NOMINAL_GHZ = 2.4               # the engine clock the published peaks are quoted at
 # HBM bytes per launch of the dominant kernels come from the committed counter profile (two rocprofv3 --pmc
 # runs of this file, FETCH_SIZE and WRITE_SIZE, each scaled by what the same counter reads for --copy-probe's
 # 1 GiB copy): its `traffic_bytes <kernel> <bytes>` rows are read at run time, so the figure printed is the
@@ -179,6 +180,8 @@ def run_config(cfg, steps, warmup, torch, dev, b1, synth, O, parity_tokens, cpu_
     wall_ms, ev_ms = timed_steps(layer, scratch, d, wl.rows, steps, warmup, torch, b1)
     per_step = spread(sampled_steps(layer, scratch, d, wl.rows, samples, warmup, torch, b1)) if samples else None
     ph = kernel_phases(layer, scratch, d, wl.rows, PREFILL_SAMPLES, b1)
+    ticks = scratch.view("clock", np.uint64, 4)  # the tile launches of the last call: shader-clock and 100 MHz ticks, FC1 then FC2
+    ph["clock_ghz"] = [float(ticks[i]) / float(ticks[i + 1]) * 0.1 if ticks[i + 1] else None for i in (0, 2)]
     after = d["out"].cpu().numpy().view(np.uint16)
     tokens = np.arange(min(parity_tokens, wl.rows))
     par = sample_parity(wl, pools, after, tokens, O)
@@ -397,6 +400,18 @@ def main():
         line["prefill"]["roofline"]["measured_mfma_TFLOPs"] = mfma_tf
         line["prefill"]["roofline"]["frac_of_measured"] = fc1_tf / mfma_tf
         line["prefill"]["roofline"]["path"]["frac_of_measured"] = tf / mfma_tf
+        # The clock the part held: under the tile kernels (one work item in the middle of each launch) and under a
+        # loop of nothing but MFMAs that lasts as long as the timed region. `peak` above is the published figure,
+        # quoted at the 2.4 GHz the part does not hold under either load; frac_at_clock prices the kernel against
+        # the matrix pipe's rate at the clock the kernel itself ran at.
+        held = probe.mfma_sustained()
+        fc1_ghz, fc2_ghz = pre["phases"]["clock_ghz"]
+        line["prefill"]["roofline"]["clock"] = {
+            "nominal_ghz": NOMINAL_GHZ, "fc1_tile_kernel_ghz": fc1_ghz, "fc2_tile_kernel_ghz": fc2_ghz,
+            "mfma_only_ghz": held["ghz_last"], "mfma_only_TFLOPs_first_launch": held["tflops_first"],
+            "mfma_only_TFLOPs_after_40_launches": held["tflops_last"]}
+        if fc1_ghz:
+            line["prefill"]["roofline"]["frac_at_clock"] = fc1_tf / (MFMA_FP8_PEAK_TFLOPS * fc1_ghz / NOMINAL_GHZ)
     if not args.no_stack:
         # configs[4] with all 48 layers resident needs about 175 GiB of HBM; without it the object says so.
         free_gib = torch.cuda.mem_get_info()[0] / 2**30

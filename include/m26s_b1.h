@@ -151,7 +151,10 @@ void m26s_b1_scratch_set_taps(m26s_b1_scratch* scratch, int on);
  * routes, 2 grouped weights, 3 groups, 4 meta words {group count, plan fault, chunk count, fc1
  * fault, quantizer fault, lowest faulting block, fc2 fault, reduce fault}, 5 intermediate payload
  * [groups*16][I], 6 its scales [groups*16][I/32], 7 y [rows*8][4096], 8/9/10 gate/up/h taps,
- * 11 chunks (16 bytes each: first group, groups, expert, zero). Returns 0, or 1 for an unknown or unallocated buffer. */
+ * 11 chunks (16 bytes each: first group, groups, expert, zero), 12 the clock record of the last call that ran
+ * the prefill-size schedule: four 64-bit words {shader-clock ticks, ticks of the fixed 100 MHz counter} over one
+ * work item in the middle of the gate/up launch, then the same of the down launch (the ratio x 0.1 is the clock
+ * in GHz the launch ran at; zeros before the first such call). Returns 0, or 1 for an unknown or unallocated buffer. */
 int m26s_b1_scratch_view(const m26s_b1_scratch* scratch, int which, void** dev_ptr, size_t* bytes);
 /* Plain copies for callers without a HIP binding of their own (synchronous). */
 int m26s_b1_copy_to_host(void* dst_host, const void* src_dev, size_t bytes);

@@ -52,6 +52,7 @@ SIGNATURES = {
 PROBE_SIGNATURES = {
     "m26p_read_bandwidth": (C.c_int, [C.c_uint64, C.c_int, _vp, C.POINTER(C.c_double), _cp, _sz]),
     "m26p_mfma_rate": (C.c_int, [C.c_int, C.c_int, _vp, C.POINTER(C.c_double), _cp, _sz]),
+    "m26p_mfma_sustained": (C.c_int, [C.c_int, C.c_int, _vp] + [C.POINTER(C.c_double)] * 4 + [_cp, _sz]),
 }
 
 _LIB = None

@@ -93,7 +93,7 @@ class Scratch:
     """Per-request device scratch and the B1 stream. b1.rs:94-118."""
 
     VIEW = dict(inverse=0, original_routes=1, grouped_weights=2, groups=3, meta=4, mid_payload=5, mid_scales=6,
-                y=7, gate=8, up=9, h=10, chunks=11)
+                y=7, gate=8, up=9, h=10, chunks=11, clock=12)
 
     def __init__(self, stream: int | None = None):
         self._h = C.c_void_p()

@@ -67,7 +67,7 @@ uint32_t tiles_for(uint32_t rows) { return rows <= 32 ? 1u : rows <= 128 ? 2u : 
 // call to call (the fault words accumulate until the next sync; the zero row and the unit scales are
 // written once); the rest is per call and may move when the slab grows.
 struct Fixed {
-    uint32_t* meta;      // kMetaWords fault / count words
+    uint32_t* meta;      // kMetaWords fault / count words; 64 bytes on, four 64-bit words of the tile launches' clock record
     uint8_t* zero_row;   // 8192 zero bytes: the activation row of a padded tile row
     uint8_t* unit_scales;  // 256 bytes of 127
 };
@@ -287,11 +287,11 @@ PlanView plan_view(const Launch& k) {
 Fc1Args fc1_args(const m26s_b1_layer* L, const Launch& k, const uint8_t* x, size_t xp, const uint8_t* xs, size_t xsp) {
     return Fc1Args{L->prepared, L->lay, plan_view(k), x, xp, xs, xsp, k.fixed.zero_row, k.fixed.unit_scales, k.ws.dq, k.ws.dqs,
                    k.taps ? k.ws.tap_gate : nullptr, k.taps ? k.ws.tap_up : nullptr, k.taps ? k.ws.tap_h : nullptr,
-                   k.ws.xg, k.ws.rowbad, k.ws.xrows, k.ws.dg};
+                   k.ws.xg, k.ws.rowbad, k.ws.xrows, k.ws.dg, reinterpret_cast<unsigned long long*>(k.fixed.meta + 16)};
 }
 Fc2Args fc2_args(const m26s_b1_layer* L, const Launch& k) {
     return Fc2Args{L->prepared, L->lay, plan_view(k), k.ws.dq, k.ws.dqs, k.fixed.zero_row, k.fixed.unit_scales, k.ws.y,
-                   uint32_t(k.ws.routes), k.ws.dg, k.ws.yrows, k.ws.rowbad};
+                   uint32_t(k.ws.routes), k.ws.dg, k.ws.yrows, k.ws.rowbad, reinterpret_cast<unsigned long long*>(k.fixed.meta + 16)};
 }
 
 // Decode-size calls: every wave streams its own weight block from HBM, activations from L2.
@@ -706,10 +706,10 @@ int m26s_b1_scratch_view(const m26s_b1_scratch* S, int which, void** dev_ptr, si
     if (!S || !dev_ptr || !bytes || !S->slab) return 1;
     const Workspace& w = S->last;
     void* const table[] = {w.inverse, w.original, w.grouped_weights, w.groups, S->fixed, w.dq, w.dqs, w.y,
-                           w.tap_gate, w.tap_up, w.tap_h, w.chunks};
+                           w.tap_gate, w.tap_up, w.tap_h, w.chunks, S->fixed + 64};
     if (which < 0 || which >= int(sizeof table / sizeof table[0]) || !table[which]) return 1;
     *dev_ptr = table[which];
-    *bytes = which == 4 ? size_t(kMetaWords) * 4 : w.bytes[which];
+    *bytes = which == 4 ? size_t(kMetaWords) * 4 : which == 12 ? 32 : w.bytes[which];
     return 0;
 }
 

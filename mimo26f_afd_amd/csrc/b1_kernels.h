@@ -709,6 +709,7 @@ struct Fc1Args {
                              // bit 8+t set where tile t holds a token in that row
     const int32_t* xrows;    // [chunk][8 tiles][16]: the token each row of each tile reads, -1 for none
     uint8_t* dg;           // the intermediate's scales in the same order, written here for FC2
+    unsigned long long* clock;  // tile schedule only, may be null: see TileClock in b1_tile.h
 };
 
 // FC1 epilogue of one wave for one activation tile: SwiGLU on the gate/up accumulators (tiles 0,1
@@ -873,6 +874,7 @@ struct Fc2Args {
     const uint8_t* dg;  // tile schedule only: the intermediate's scales in MFMA lane order (see Fc1Args)
     const int32_t* yrows;  // tile schedule only, [chunk][8 tiles][16]: the route (row of y) of each row, -1 for none
     const uint32_t* rowbad;  // tile schedule only: as in Fc1Args (bit 8+t: tile t holds a token in that row)
+    unsigned long long* clock;  // tile schedule only, may be null: see TileClock in b1_tile.h
 };
 
 // FC2 epilogue of one wave: unweighted FP32 rows back to y[original route].

@@ -479,6 +479,23 @@ __device__ __forceinline__ void fc2_tile_body(const Fc2Args& a, const Chunk ch, 
     if (lost) atomicOr(&a.plan.meta[kFc2Fault], 5u);
 }
 
+// The clock a tile launch ran at. The shader clock of these parts is not a constant of the launch: under the
+// load of the tile kernels the power management takes it well below what the same part holds on a loop of
+// nothing but MFMAs, so a cycle count says little without it. The workgroup of the middle chunk's first column
+// set (every compute unit busy around it, once the call is large enough to fill them) reads the shader-clock
+// counter and the fixed 100 MHz counter at both ends of its item and leaves the two differences in clock[0..1];
+// their ratio x 0.1 is the clock in GHz.
+struct TileClock {
+    unsigned long long shader, fixed;
+    __device__ __forceinline__ void start() { shader = __builtin_amdgcn_s_memtime(), fixed = __builtin_amdgcn_s_memrealtime(); }
+    __device__ __forceinline__ void stop(unsigned long long* out, bool mine) const {
+        if (out && mine && threadIdx.x == 0) {
+            out[0] = __builtin_amdgcn_s_memtime() - shader;
+            out[1] = __builtin_amdgcn_s_memrealtime() - fixed;
+        }
+    }
+};
+
 // Work item of a tile workgroup. Workgroups are handed to the eight XCDs in turn, each with an L2 of
 // its own: the `columns` workgroups of one chunk all take ids of one residue mod 8, so a chunk's
 // activation rows enter one L2 only. FC2 hands an XCD runs of two neighbouring chunks: chunks are in
@@ -506,6 +523,8 @@ template <class S>
 __global__ void __launch_bounds__(S::kThreads, 8 / S::kWaves) fc1_tile_kernel(Fc1Args a) {
     extern __shared__ __align__(16) uint8_t lds[];
     uint32_t* meta = a.plan.meta;
+    TileClock clock;
+    clock.start();
     const TileItem it = tile_item<kFc1Run>(a.lay.inter / (32 * S::kWaves));
     const uint32_t c = it.chunk;
     const uint32_t lane = threadIdx.x & 63, wv = threadIdx.x >> 6, cb = it.column * S::kWaves + wv;
@@ -529,6 +548,7 @@ __global__ void __launch_bounds__(S::kThreads, 8 / S::kWaves) fc1_tile_kernel(Fc
     else if (ch.groups == 2) fc1_body<2>(a, ch, cb, lane);
     else if (ch.groups <= 4) fc1_tile_body<S, 4>(a, ch, c, cb, wv, lane, lds, token4);
     else fc1_tile_body<S, 8>(a, ch, c, cb, wv, lane, lds, token8);
+    clock.stop(a.clock, c == head.meta[kChunkCount] / 2 && it.column == 0);
 }
 
 // One workgroup per (chunk, 64 * kWaves output columns). ONE: the layer holds one rank's share (I = 512, a single
@@ -537,6 +557,8 @@ template <class S, bool ONE>
 __global__ void __launch_bounds__(S::kThreads, 8 / S::kWaves) fc2_tile_kernel(Fc2Args a) {
     extern __shared__ __align__(16) uint8_t lds[];
     uint32_t* meta = a.plan.meta;
+    TileClock clock;
+    clock.start();
     const TileItem it = tile_item<kFc2Run>(kHidden / (64 * S::kWaves));
     const uint32_t c = it.chunk;
     const uint32_t lane = threadIdx.x & 63, wv = threadIdx.x >> 6, ob = it.column * S::kWaves + wv;
@@ -553,6 +575,7 @@ __global__ void __launch_bounds__(S::kThreads, 8 / S::kWaves) fc2_tile_kernel(Fc
     else if (ch.groups == 2) fc2_body<2>(a, ch, ob, lane);
     else if (ch.groups <= 4) fc2_tile_body<S, 4, ONE>(a, ch, c, ob, wv, lane, lds, verdict);
     else fc2_tile_body<S, 8, ONE>(a, ch, c, ob, wv, lane, lds, verdict);
+    clock.stop(a.clock ? a.clock + 2 : nullptr, c == head.meta[kChunkCount] / 2 && it.column == 0);
 }
 
 }  // namespace m26g

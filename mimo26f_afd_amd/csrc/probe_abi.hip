@@ -1,6 +1,7 @@
 // Measurement aids: what this GPU sustains on the two rooflines the FFN is priced against
 // (declared in include/m26_probe.h).
 #include <hip/hip_runtime.h>
+#include <vector>
 #include <stdint.h>
 #include <stdio.h>
 #include "../../include/m26_probe.h"
@@ -46,8 +47,11 @@ __global__ void __launch_bounds__(256) read_kernel(const v4i* __restrict__ p, si
 
 // 32 independent accumulators per wave (4 weight tiles x 8 activation tiles, the tile kernels'
 // shape); the accumulator is tied so no copy is issued between the MFMAs.
-__global__ void __launch_bounds__(256, 2) mfma_kernel(const v4i* w, const v8i* x, float* out, int iters) {
+// `clock`, when given, receives from one workgroup in the middle of the grid what its first wave read before and
+// after its loop: {shader-clock ticks, ticks of the fixed 100 MHz counter}.
+__global__ void __launch_bounds__(256, 2) mfma_kernel(const v4i* w, const v8i* x, float* out, int iters, unsigned long long* clock) {
     const int lane = threadIdx.x & 63;
+    const unsigned long long t0 = __builtin_amdgcn_s_memtime(), r0 = __builtin_amdgcn_s_memrealtime();
     v4i a[4];
     v8i b[8];
 #pragma unroll
@@ -70,6 +74,10 @@ __global__ void __launch_bounds__(256, 2) mfma_kernel(const v4i* w, const v8i* x
                              : "+a"(acc[t][tt]) : "v"(a[t]), "v"(b[tt]), "v"(sa), "v"(sb));
     }
     asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15" ::: "memory");  // the last MFMAs retire before their results are read
+    if (clock && blockIdx.x == gridDim.x / 2 && threadIdx.x == 0) {
+        clock[0] = __builtin_amdgcn_s_memtime() - t0;
+        clock[1] = __builtin_amdgcn_s_memrealtime() - r0;
+    }
     float s = 0.f;
 #pragma unroll
     for (int t = 0; t < 4; ++t)
@@ -135,7 +143,7 @@ extern "C" int m26p_mfma_rate(int iters, int reps, void* stream, double* tflops,
     const double flops = double(grid) * (threads / 64) * double(iters) * 32.0 * (2.0 * 16 * 16 * 128);
     for (int r = 0; r <= reps; ++r) {
         M26P_TRY(hipEventRecord(ev.a, s), "hipEventRecord");
-        mfma_kernel<<<grid, threads, 0, s>>>(static_cast<const v4i*>(w.p), static_cast<const v8i*>(x.p), static_cast<float*>(out.p), iters);
+        mfma_kernel<<<grid, threads, 0, s>>>(static_cast<const v4i*>(w.p), static_cast<const v8i*>(x.p), static_cast<float*>(out.p), iters, nullptr);
         M26P_TRY(hipEventRecord(ev.b, s), "hipEventRecord");
         M26P_TRY(hipEventSynchronize(ev.b), "mfma kernel");
         float ms = 0.f;
@@ -143,5 +151,44 @@ extern "C" int m26p_mfma_rate(int iters, int reps, void* stream, double* tflops,
         if (r && ms > 0.f && flops / (ms * 1e-3) / 1e12 > best) best = flops / (ms * 1e-3) / 1e12;
     }
     *tflops = best;
+    return 0;
+}
+
+extern "C" int m26p_mfma_sustained(int iters, int launches, void* stream, double* tflops_first, double* tflops_last,
+                                   double* ghz_first, double* ghz_last, char* err, size_t errlen) {
+    if (!tflops_first || !tflops_last || !ghz_first || !ghz_last || iters < 1 || iters > 100000 || launches < 2 || launches > 1000)
+        return fail(err, errlen, 1, "mfma_sustained: iters 1..100000, launches 2..1000");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const int grid = 2048, threads = 256;
+    Buffer w, x, out, clock;
+    M26P_TRY(hipMalloc(&w.p, 4 * 64 * 16), "hipMalloc");
+    M26P_TRY(hipMalloc(&x.p, 8 * 64 * 32), "hipMalloc");
+    M26P_TRY(hipMalloc(&out.p, size_t(grid) * threads * 4), "hipMalloc");
+    M26P_TRY(hipMalloc(&clock.p, size_t(launches) * 16), "hipMalloc");
+    std::vector<hipEvent_t> ev(size_t(launches) + 1, nullptr);
+    struct Drop { std::vector<hipEvent_t>& e; ~Drop() { for (hipEvent_t v : e) if (v) (void)hipEventDestroy(v); } } drop{ev};
+    for (hipEvent_t& e : ev) M26P_TRY(hipEventCreate(&e), "hipEventCreate");
+    fill_kernel<<<4, 256, 0, s>>>(static_cast<uint32_t*>(w.p), 4 * 64 * 4, 0xffffffffu);
+    fill_kernel<<<16, 256, 0, s>>>(static_cast<uint32_t*>(x.p), 8 * 64 * 8, 0xf7f7f7f7u);
+    M26P_TRY(hipStreamSynchronize(s), "fill");
+    M26P_TRY(hipEventRecord(ev[0], s), "hipEventRecord");
+    for (int r = 0; r < launches; ++r) {  // back to back, nothing between them but an event
+        mfma_kernel<<<grid, threads, 0, s>>>(static_cast<const v4i*>(w.p), static_cast<const v8i*>(x.p), static_cast<float*>(out.p), iters,
+                                             static_cast<unsigned long long*>(clock.p) + 2 * r);
+        M26P_TRY(hipEventRecord(ev[size_t(r) + 1], s), "hipEventRecord");
+    }
+    M26P_TRY(hipEventSynchronize(ev[size_t(launches)]), "mfma kernels");
+    std::vector<unsigned long long> ticks(size_t(launches) * 2);
+    M26P_TRY(hipMemcpy(ticks.data(), clock.p, ticks.size() * 8, hipMemcpyDeviceToHost), "hipMemcpy");
+    const double flops = double(grid) * (threads / 64) * double(iters) * 32.0 * (2.0 * 16 * 16 * 128);
+    auto rate = [&](int r, double* tf, double* ghz) -> hipError_t {
+        float ms = 0.f;
+        const hipError_t e = hipEventElapsedTime(&ms, ev[size_t(r)], ev[size_t(r) + 1]);
+        *tf = ms > 0.f ? flops / (ms * 1e-3) / 1e12 : 0.0;
+        *ghz = ticks[2 * size_t(r) + 1] ? double(ticks[2 * size_t(r)]) / double(ticks[2 * size_t(r) + 1]) * 0.1 : 0.0;
+        return e;
+    };
+    M26P_TRY(rate(0, tflops_first, ghz_first), "hipEventElapsedTime");
+    M26P_TRY(rate(launches - 1, tflops_last, ghz_last), "hipEventElapsedTime");
     return 0;
 }

@@ -26,3 +26,13 @@ def read_bandwidth_gbps(nbytes: int = 4 << 30, reps: int = 5, stream: int | None
 def mfma_rate_tflops(iters: int = 2000, reps: int = 3, stream: int | None = None) -> float:
     """Best of `reps` runs of nothing but the GEMMs' block-scaled MFMA, in TFLOP/s."""
     return _run("m26p_mfma_rate", iters, reps, stream)
+
+
+def mfma_sustained(iters: int = 2000, launches: int = 40, stream: int | None = None) -> dict:
+    """`launches` runs of the MFMA-only kernel back to back: rate and shader clock of the first and of the last."""
+    v = [C.c_double(0.0) for _ in range(4)]
+    buf = C.create_string_buffer(256)
+    rc = load_probe().m26p_mfma_sustained(iters, launches, stream, *[C.byref(x) for x in v], buf, 256)
+    if rc != 0:
+        raise ProbeError(f"m26p_mfma_sustained: rc {rc}: {buf.value.decode('utf-8', 'replace')}")
+    return dict(tflops_first=v[0].value, tflops_last=v[1].value, ghz_first=v[2].value, ghz_last=v[3].value)

@@ -230,6 +230,12 @@ def test_tile_schedule_at_full_intermediate_every_row(scratch, full_layer):
     assert per_row.max() <= MAX_ABS, ("worst row", int(per_row.argmax()), float(per_row.max()))
     _, bf2, pf2 = run_ffn_dev(layer, scratch, wl)
     assert np.array_equal(bf2, bf) and np.array_equal(pf2.view(np.uint32), pf.view(np.uint32))
+    # The clock record of the two tile launches: ticks of the shader clock and of the fixed 100 MHz counter over
+    # one work item each (the middle chunk's); an item lasts microseconds to tens of them and the clock lies
+    # between 1 and 2.4 GHz.
+    ticks = scratch.view("clock", np.uint64, 4)
+    for shader, fixed in (ticks[:2], ticks[2:]):
+        assert 200 < fixed < 100_000 and 1.0 < float(shader) / float(fixed) * 0.1 < 2.6, ticks
 
 
 def test_prefill_chunk_properties_and_sampled_parity(full_layer):

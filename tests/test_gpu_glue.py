@@ -168,3 +168,10 @@ def test_roofline_probes_report_plausible_rates():
         probe.read_bandwidth_gbps(12345, 1)
     with pytest.raises(probe.ProbeError):
         probe.mfma_rate_tflops(0, 1)
+    held = probe.mfma_sustained(500, 4)  # the same loop four times back to back, with the clock it ran at
+    assert 1600 < held["tflops_first"] < 5500 and 1600 < held["tflops_last"] < 5500, held
+    assert 1.0 < held["ghz_first"] < 2.6 and 1.0 < held["ghz_last"] < 2.6, held  # 2.4 GHz is the part's ceiling
+    # the matrix pipe's rate follows the clock: 2 x 16 x 16 x 128 flops per MFMA, 32 cycles each, 1024 SIMDs
+    assert 0.85 < held["tflops_last"] / (held["ghz_last"] * 1e9 * 1024 * 65536 / 32 / 1e12) <= 1.02, held
+    with pytest.raises(probe.ProbeError):
+        probe.mfma_sustained(500, 1)
