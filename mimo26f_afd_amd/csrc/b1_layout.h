@@ -30,7 +30,8 @@
 // consecutive k-steps through the MFMA's scale byte select.
 // (Version 1 kept every block's k-steps together, [cb][ks]: a wave streamed one contiguous run of 128 or 64 KB.
 // A bare streaming kernel whose workgroups read their four waves' k-steps back to back reaches 6.8-6.9 TB/s
-// where one contiguous run per wave reaches 6.2-6.4; the decode step became 2.5 % shorter with this order.)
+// where one contiguous run per wave reaches 6.2-6.4; the decode step became 1.5 % shorter with this order (same box,
+// interleaved runs).)
 #pragma once
 #include <stdint.h>
 #include <stddef.h>
