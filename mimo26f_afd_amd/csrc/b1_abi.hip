@@ -302,7 +302,7 @@ void launch_direct(const m26s_b1_layer* L, const Launch& k, const Fc1Args& f1, c
     fc2_kernel<NT><<<dim3(16, k.ws.chunk_cap), 256, 0, k.stream>>>(f2);
     mark(k.fc2_done, k.stream);
 }
-// Prefill-size calls: workgroups that share each chunk's activation tiles through LDS, two per compute unit.
+// Prefill-size calls: workgroups that share each chunk's activation tiles through LDS, one of eight waves per compute unit.
 void launch_tiles(const m26s_b1_layer* L, const Launch& k, const Fc1Args& f1, const Fc2Args& f2) {
     gather_scales_kernel<<<k.ws.chunk_cap, 256, 0, k.stream>>>(f1.plan, f1.xs, f1.xs_pitch, reinterpret_cast<uint32_t*>(k.ws.xg),
                                                               k.ws.rowbad, k.ws.xrows, k.ws.yrows);
