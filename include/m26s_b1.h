@@ -95,10 +95,13 @@ int m26s_b1_ffn_dev(const m26s_b1_layer* layer, m26s_b1_scratch* scratch, const 
                     const int32_t* ids_dev, const float* weights_dev, uint32_t rows,
                     uint16_t* bf16_out_dev, float* partial_dev, float* ms, char* err, size_t errlen);
 /* Same work, enqueued only: returns after the launches. Faults of every call since the last
- * m26s_b1_scratch_sync accumulate and are reported there: once a call's routes have been rejected or
- * one of its stages has faulted, the later calls enqueued on the scratch before that sync compute
- * nothing, and the sync returns the first fault's code (3 before 4). The call puts its kernels on the
- * stream and nothing else (no events: the synchronous entries record theirs only when ms is given). */
+ * m26s_b1_scratch_sync accumulate and are reported there as the OR of the calls' fault words, routes
+ * before numerics (3 before 4). What a fault stops: a rejected plan stops every stage of its own call and
+ * of every later call enqueued before that sync; a fault of FC1 or of the quantizer stops FC2 and the
+ * combine of its own and of later calls, but not their plan or FC1; an FC2 or combine fault stops
+ * nothing that follows. After a nonzero sync every output written since the previous sync is invalid. The
+ * call puts its kernels on the stream and nothing else (no events: the synchronous entries record theirs
+ * only when ms is given). */
 int m26s_b1_ffn_enqueue(const m26s_b1_layer* layer, m26s_b1_scratch* scratch, const uint8_t* payload_dev,
                         size_t payload_pitch, const uint8_t* scales_dev, size_t scales_pitch,
                         const int32_t* ids_dev, const float* weights_dev, uint32_t rows,
@@ -147,6 +150,26 @@ int m26s_b1_reduce_dev(const float* y_dev, const float* weights_dev, uint32_t ro
 
 /* With taps on, the next FFN calls also keep FP32 gate / up / h of every grouped row. */
 void m26s_b1_scratch_set_taps(m26s_b1_scratch* scratch, int on);
+/* Switches of a scratch, for the calls made on it afterwards. Returns 0, 1 for a bad handle or option, 2 for
+ * a runtime error.
+ *   TAPS              as m26s_b1_scratch_set_taps.
+ *   SEPARATE_COMBINE  the router-weighted combine runs as a launch of its own behind FC2
+ *                     (crates/mimo26-spark/kernels/b1_serve.cu:502-515 launches it so). By default FC2 does it:
+ *                     the wave that writes a token's eighth per-route row sums the eight, in slot order, so
+ *                     both forms give the same bits. Layers on the conforming arm always combine separately.
+ *   BF16_ROUTE_ROWS   the reference's opt-in MIMO26_B1_Y=bf16 (b1_serve.cu:98-143,400-405; the store rule of
+ *                     crates/mimo26-expert/kernels/b1/connected.cu:41-44): FC2 keeps its per-route rows as
+ *                     BF16 bits instead of FP32 and the combine widens them. A numerical-mode change, never
+ *                     the default; a scratch is created with it on when the environment holds MIMO26_B1_Y=bf16.
+ *                     View 7 then holds uint16 rows.
+ *   GUARDS            test aid (the counterpart of crates/mimo26-expert/tests/b1_core/primitive.cu:23-40):
+ *                     every internal array is followed, and the first preceded, by at least 256 bytes of 0xa5,
+ *                     written before each call and read back by m26s_b1_scratch_check_guards. */
+enum { M26S_B1_OPT_TAPS = 0, M26S_B1_OPT_SEPARATE_COMBINE = 1, M26S_B1_OPT_BF16_ROUTE_ROWS = 2, M26S_B1_OPT_GUARDS = 3 };
+int m26s_b1_scratch_set_option(m26s_b1_scratch* scratch, int option, int value);
+/* Waits for the scratch's stream and reads every red zone back: 0 intact, 1 guards not enabled or no call made,
+ * 2 runtime error, 4 a zone holds a byte other than 0xa5 (err names the zone and the offset). */
+int m26s_b1_scratch_check_guards(m26s_b1_scratch* scratch, char* err, size_t errlen);
 /* Device address and byte size of an internal buffer after a call. which: 0 inverse, 1 original
  * routes, 2 grouped weights, 3 groups, 4 meta words {group count, plan fault, chunk count, fc1
  * fault, quantizer fault, lowest faulting block, fc2 fault, reduce fault}, 5 intermediate payload
@@ -161,6 +184,8 @@ int m26s_b1_copy_to_host(void* dst_host, const void* src_dev, size_t bytes);
 int m26s_b1_copy_to_device(void* dst_dev, const void* src_host, size_t bytes);
 void* m26s_b1_device_alloc(size_t bytes);
 void m26s_b1_device_free(void* dev_ptr);
+/* Free and total bytes of the current GPU's memory (hipMemGetInfo): 0, 1 for a null argument, 2 for a runtime error. */
+int m26s_b1_device_memory(size_t* free_bytes, size_t* total_bytes);
 
 #ifdef __cplusplus
 }

@@ -40,6 +40,9 @@ SIGNATURES = {
     "m26s_b1_quantize_dev": (C.c_int, [_vp, C.c_uint64, _vp, _vp, _vp, _cp, _sz]),
     "m26s_b1_reduce_dev": (C.c_int, [_vp, _vp, C.c_uint32, _vp, _vp, _vp, _cp, _sz]),
     "m26s_b1_scratch_set_taps": (None, [_vp, C.c_int]),
+    "m26s_b1_scratch_set_option": (C.c_int, [_vp, C.c_int, C.c_int]),
+    "m26s_b1_scratch_check_guards": (C.c_int, [_vp, _cp, _sz]),
+    "m26s_b1_device_memory": (C.c_int, [C.POINTER(_sz), C.POINTER(_sz)]),
     "m26s_b1_scratch_stream": (_vp, [_vp]),
     "m26s_b1_scratch_view": (C.c_int, [_vp, C.c_int, C.POINTER(_vp), C.POINTER(_sz)]),
     "m26s_b1_copy_to_host": (C.c_int, [_vp, _vp, _sz]),

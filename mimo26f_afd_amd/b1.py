@@ -103,8 +103,23 @@ class Scratch:
         else:
             _raise(load().m26s_b1_scratch_new_on(stream, C.byref(self._h), buf, ERRLEN), buf)
 
+    OPTION = dict(taps=0, separate_combine=1, bf16_route_rows=2, guards=3)
+
     def set_taps(self, on: bool) -> None:
         load().m26s_b1_scratch_set_taps(self._h, 1 if on else 0)
+
+    def set_option(self, name: str, on: bool) -> None:
+        """Switches for the calls that follow: 'separate_combine' (the combine as a launch of its own instead of
+        inside FC2; same bits), 'bf16_route_rows' (the reference's opt-in MIMO26_B1_Y=bf16 numerical mode),
+        'guards' (red zones around every internal array, read back by check_guards), 'taps'."""
+        rc = load().m26s_b1_scratch_set_option(self._h, self.OPTION[name], 1 if on else 0)
+        if rc:
+            raise B1Error(rc, f"b1 scratch: option {name} refused")
+
+    def check_guards(self) -> None:
+        """Waits for the stream and raises when a red zone of the last call's workspace was written to."""
+        buf = _err()
+        _raise(load().m26s_b1_scratch_check_guards(self._h, buf, ERRLEN), buf)
 
     @property
     def stream(self) -> int:
@@ -222,6 +237,14 @@ def quantize_dev(h_dev, elements, payload_dev, scales_dev, faults_dev) -> None:
 def reduce_dev(y_dev, weights_dev, rows, partial_dev, bf16_dev, fault_dev) -> None:
     buf = _err()
     _raise(load().m26s_b1_reduce_dev(y_dev, weights_dev, rows, partial_dev, bf16_dev, fault_dev, buf, ERRLEN), buf)
+
+
+def device_memory() -> tuple[int, int]:
+    """(free, total) bytes of the current GPU's memory."""
+    free, total = C.c_size_t(), C.c_size_t()
+    if load().m26s_b1_device_memory(C.byref(free), C.byref(total)):
+        raise B1Error(2, "b1: memory query failed")
+    return int(free.value), int(total.value)
 
 
 class DeviceBuffer:

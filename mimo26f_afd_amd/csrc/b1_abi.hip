@@ -6,9 +6,11 @@
 // workgroups leave on the device-side counts), the intermediate quantizer is fused into FC1, and a
 // layer with exceptional weight scales runs the conforming arm of b1_conform.h.
 #include <hip/hip_runtime.h>
+#include <atomic>
 #include <chrono>
 #include <cstdarg>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <new>
 #include <vector>
@@ -72,7 +74,7 @@ struct Fixed {
     uint8_t* unit_scales;  // 256 bytes of 127
 };
 constexpr size_t kFixedBytes = 256 + 8192 + 256;
-Fixed fixed_at(uint8_t* base) {
+__host__ __device__ inline Fixed fixed_at(uint8_t* base) {
     return Fixed{reinterpret_cast<uint32_t*>(base), base + 256, base + 256 + 8192};
 }
 __global__ void fixed_init_kernel(uint8_t* base) {  // a kernel, not a memset: a caller may be recording a graph
@@ -80,18 +82,29 @@ __global__ void fixed_init_kernel(uint8_t* base) {  // a kernel, not a memset: a
         base[i] = i >= 256 + 8192 ? uint8_t(127) : (i / 4 == kQuantWhere ? uint8_t(0xff) : uint8_t(0));
 }
 
+__global__ void arm_plan_work_kernel(uint32_t* work) {
+    if (threadIdx.x < 4) work[threadIdx.x] = 0xffffffffu;
+}
+
 struct Shape {
     uint32_t rows, inter;
     bool taps, host_io, conforming;
+    bool fused;   // the combine runs inside FC2 (completion counts per token and 64 columns), not as a launch of its own
+    bool y_bf16;  // per-route rows kept as BF16 bits
+    bool guards;  // every array is followed (and the first preceded) by a red zone of 0xa5 bytes
 };
+constexpr int kMaxZones = 32;
+constexpr uint8_t kGuardByte = 0xa5;
+struct Zone { uint64_t at, bytes; };  // relative to the slab
 struct Workspace {
-    uint32_t* plan_work;  // the wide planner's histograms (always first: its header word is armed when the slab moves)
+    uint32_t* plan_work;  // the wide planner's histograms (its header word is armed when the slab moves)
     int32_t *inverse, *original;
     float* grouped_weights;
     Group* groups;
     Chunk* chunks;
     uint8_t *dq, *dqs;
     float* y;
+    uint32_t* done;    // fused combine: [rows][64] completion counts
     uint8_t *xg, *dg;  // tile schedule: activation scales in MFMA lane order
     uint32_t* rowbad;
     int32_t *xrows, *yrows;
@@ -104,6 +117,8 @@ struct Workspace {
     size_t total;
     uint32_t tiles, chunk_cap, group_cap;
     uint64_t routes, route_cap;
+    Zone zone[kMaxZones];
+    int zones;
 };
 constexpr size_t kPlanWorkBytes = wide_plan_words(kMaxRows * kTopk) * 4;
 
@@ -111,9 +126,15 @@ constexpr size_t kPlanWorkBytes = wide_plan_words(kMaxRows * kTopk) * 4;
 Workspace carve(uint8_t* base, const Shape& s) {
     Workspace w{};
     size_t at = 0;
+    auto zone = [&](size_t from, size_t upto) {
+        if (w.zones < kMaxZones) w.zone[w.zones++] = Zone{from, upto - from};
+    };
+    if (s.guards) zone(0, at = 256);
     auto take = [&](size_t bytes) {
         uint8_t* p = base ? base + at : nullptr;
+        const size_t end = at + ((bytes + 3) & ~size_t(3));
         at += (bytes + 255) & ~size_t(255);
+        if (s.guards) zone(end, at += 256);  // from the array's last word to 256 bytes past its padded end
         return p;
     };
     w.tiles = tiles_for(s.rows);
@@ -133,7 +154,8 @@ Workspace carve(uint8_t* base, const Shape& s) {
     w.chunks = reinterpret_cast<Chunk*>(take(w.bytes[11] = grid_chunks * sizeof(Chunk)));
     w.dq = take(w.bytes[5] = gcap * 16 * I);
     w.dqs = take(w.bytes[6] = gcap * 16 * I / 32);
-    w.y = reinterpret_cast<float*>(take(w.bytes[7] = w.routes * kHidden * 4));
+    w.y = reinterpret_cast<float*>(take(w.bytes[7] = w.routes * kHidden * (s.y_bf16 ? 2 : 4)));
+    if (s.fused) w.done = reinterpret_cast<uint32_t*>(take(size_t(s.rows) * kDoneBlocks * 4));
     if (w.tiles > 2 && !s.conforming) {
         w.xg = take(ccap * gathered_scale_bytes(kHidden));
         w.dg = take(ccap * gathered_scale_bytes(s.inter));
@@ -157,8 +179,18 @@ Workspace carve(uint8_t* base, const Shape& s) {
     return w;
 }
 
+// Red zones (test aid): filled before every call when the scratch asks for them, read back by
+// m26s_b1_scratch_check_guards. The counterpart of the reference's guarded test buffers
+// (crates/mimo26-expert/tests/b1_core/primitive.cu:23-40).
+struct ZoneTable { Zone zone[kMaxZones]; int zones; };
+__global__ void fill_zones_kernel(uint8_t* base, ZoneTable t) {
+    if (int(blockIdx.x) >= t.zones) return;
+    const Zone z = t.zone[blockIdx.x];
+    for (uint64_t i = threadIdx.x; i < z.bytes; i += blockDim.x) base[z.at + i] = kGuardByte;
+}
+
 // Kernels whose dynamic LDS passes 64 KB need the limit raised once per process.
-bool lds_ready = false;
+std::atomic<bool> lds_ready{false};  // idempotent: threads that race set the same attributes
 using TileS = PrefillTile;
 hipError_t raise_lds_limits() {
     if (lds_ready) return hipSuccess;
@@ -194,7 +226,7 @@ struct m26s_b1_scratch {
     uint8_t* slab = nullptr;
     size_t slab_bytes = 0;
     Workspace last{};  // of the latest call, for the views
-    bool taps = false;
+    bool taps = false, separate_combine = false, y_bf16 = false, guards = false;
     uint32_t last_rows = 0;
     uint8_t* bounce = nullptr;  // page-locked host staging for callers whose own arrays are pageable
     size_t bounce_bytes = 0;
@@ -203,15 +235,34 @@ struct m26s_b1_scratch {
 namespace {
 
 // The slab only grows. Growing it frees the old one, which waits for the device: calls still in flight on it finish first.
-int fit_slab(m26s_b1_scratch* S, size_t bytes, Outcome& out) {
+int fit_slab(m26s_b1_scratch* S, size_t bytes, bool& grew, Outcome& out) {
+    grew = false;
     if (bytes <= S->slab_bytes) return 0;
     if (S->slab) (void)hipFree(S->slab);
     S->slab = nullptr;
     S->slab_bytes = 0;
     M26G_TRY(out, hipMalloc(reinterpret_cast<void**>(&S->slab), bytes), "b1 workspace alloc");
     S->slab_bytes = bytes;
-    // The wide planner's first word is its fault key, armed to "none"; its scan re-arms it after every call.
-    M26G_TRY(out, hipMemsetAsync(S->slab, 0xff, 16, S->stream), "b1 workspace arm");
+    grew = true;
+    return 0;
+}
+
+Shape shape_of(const m26s_b1_layer* L, const m26s_b1_scratch* S, uint32_t rows, bool host_io) {
+    const bool conforming = !L->all_normal;
+    return Shape{rows, L->lay.inter, S->taps, host_io, conforming, !S->separate_combine && !conforming, S->y_bf16, S->guards};
+}
+
+// Sizes the slab for the call and lays the call's arrays out in it (S->last).
+int ready_workspace(m26s_b1_scratch* S, const Shape& shape, Outcome& out) {
+    bool grew = false;
+    if (const int rc = fit_slab(S, carve(nullptr, shape).total, grew, out)) return rc;
+    S->last = carve(S->slab, shape);
+    if (grew) {
+        // The wide planner's first word is its fault key, armed to "none"; its scan re-arms it after every call.
+        // A kernel, not a memset: the stream may be the caller's, and the caller may be recording a graph.
+        arm_plan_work_kernel<<<1, 64, 0, S->stream>>>(S->last.plan_work);
+        M26G_TRY(out, hipGetLastError(), "b1 workspace arm");
+    }
     return 0;
 }
 
@@ -251,6 +302,9 @@ int scratch_build(hipStream_t stream, bool own, m26s_b1_scratch** made, Outcome&
     if (!S) return out.fail(1, "b1 scratch: host allocation failed");
     S->stream = stream;
     S->own_stream = own;
+    // The reference's opt-in switch for BF16 per-route rows (crates/mimo26-spark/kernels/b1_serve.cu:402-405).
+    const char* y_mode = std::getenv("MIMO26_B1_Y");
+    S->y_bf16 = y_mode && std::strcmp(y_mode, "bf16") == 0;
     hipError_t e = own ? hipStreamCreateWithFlags(&S->stream, hipStreamNonBlocking) : hipSuccess;
     for (hipEvent_t* ev : {&S->begun, &S->planned, &S->fc1_done, &S->fc2_done, &S->ended})
         if (e == hipSuccess) e = hipEventCreate(ev);
@@ -274,14 +328,14 @@ struct Launch {
     hipStream_t stream;
     Fixed fixed;
     Workspace ws;
-    bool taps;
+    bool taps, y_bf16;
     hipEvent_t planned, fc1_done, fc2_done;  // null: not timed
 };
 
 void mark(hipEvent_t ev, hipStream_t st) { if (ev) (void)hipEventRecord(ev, st); }
 
 PlanView plan_view(const Launch& k) {
-    return PlanView{k.ws.inverse, k.ws.original, k.ws.grouped_weights, k.ws.groups, k.ws.chunks, k.fixed.meta};
+    return PlanView{k.ws.inverse, k.ws.original, k.ws.grouped_weights, k.ws.groups, k.ws.chunks, k.fixed.meta, k.ws.done};
 }
 
 Fc1Args fc1_args(const m26s_b1_layer* L, const Launch& k, const uint8_t* x, size_t xp, const uint8_t* xs, size_t xsp) {
@@ -289,9 +343,10 @@ Fc1Args fc1_args(const m26s_b1_layer* L, const Launch& k, const uint8_t* x, size
                    k.taps ? k.ws.tap_gate : nullptr, k.taps ? k.ws.tap_up : nullptr, k.taps ? k.ws.tap_h : nullptr,
                    k.ws.xg, k.ws.rowbad, k.ws.xrows, k.ws.dg, reinterpret_cast<unsigned long long*>(k.fixed.meta + 16)};
 }
-Fc2Args fc2_args(const m26s_b1_layer* L, const Launch& k) {
+Fc2Args fc2_args(const m26s_b1_layer* L, const Launch& k, const float* w, uint16_t* bf16_out, float* partial) {
     return Fc2Args{L->prepared, L->lay, plan_view(k), k.ws.dq, k.ws.dqs, k.fixed.zero_row, k.fixed.unit_scales, k.ws.y,
-                   uint32_t(k.ws.routes), k.ws.dg, k.ws.yrows, k.ws.rowbad, reinterpret_cast<unsigned long long*>(k.fixed.meta + 16)};
+                   uint32_t(k.ws.routes), k.ws.dg, k.ws.yrows, k.ws.rowbad, reinterpret_cast<unsigned long long*>(k.fixed.meta + 16),
+                   w, bf16_out, partial, k.y_bf16};
 }
 
 // Decode-size calls: every wave streams its own weight block from HBM, activations from L2.
@@ -328,7 +383,7 @@ hipError_t launch_ffn(const m26s_b1_layer* L, const Launch& k, const uint8_t* x,
     const uint32_t nt = k.ws.tiles, routes = uint32_t(k.ws.routes);
     if (rows > kWidePlanFrom) {  // several compute units share the scatter (b1_kernels.h, "Stage 1 for large calls")
         const uint32_t wide = wide_plan_groups(routes);
-        plan_count_kernel<<<wide, kPlanThreads, 0, k.stream>>>(ids, w, rows, L->resident, k.ws.plan_work);
+        plan_count_kernel<<<wide, kPlanThreads, 0, k.stream>>>(ids, w, rows, L->resident, k.ws.plan_work, k.ws.done);
         plan_scan_kernel<<<1, kPlanThreads, 0, k.stream>>>(routes, k.ws.plan_work, pv, nt);
         plan_place_kernel<<<wide, kPlanThreads, 0, k.stream>>>(ids, w, rows, k.ws.plan_work, pv, k.taps);
     } else {
@@ -338,15 +393,16 @@ hipError_t launch_ffn(const m26s_b1_layer* L, const Launch& k, const uint8_t* x,
     if (e != hipSuccess) return e;
     mark(k.planned, k.stream);
     const Fc1Args f1 = fc1_args(L, k, x, xp, xs, xsp);
-    const Fc2Args f2 = fc2_args(L, k);
+    const Fc2Args f2 = fc2_args(L, k, w, bf16_out, partial);
     if (!L->all_normal) launch_conforming(L, k, f1, f2);
     else if (nt == 1) launch_direct<1>(L, k, f1, f2);
     else if (nt == 2) launch_direct<2>(L, k, f1, f2);
     else launch_tiles(L, k, f1, f2);
-    if ((e = hipGetLastError()) != hipSuccess) return e;
+    if ((e = hipGetLastError()) != hipSuccess || k.ws.done) return e;  // with completion counts FC2 has summed the rows itself
     const uint64_t n4 = uint64_t(rows) * (kHidden / 4);
     const uint32_t blocks = uint32_t(n4 / 256 < 65536 ? (n4 + 255) / 256 : 65536);
-    reduce_kernel<<<blocks, 256, 0, k.stream>>>(k.ws.y, w, rows, partial, bf16_out, k.fixed.meta + kReduceFault, k.fixed.meta);
+    if (k.y_bf16) reduce_kernel<true><<<blocks, 256, 0, k.stream>>>(k.ws.y, w, rows, partial, bf16_out, k.fixed.meta + kReduceFault, k.fixed.meta);
+    else reduce_kernel<false><<<blocks, 256, 0, k.stream>>>(k.ws.y, w, rows, partial, bf16_out, k.fixed.meta + kReduceFault, k.fixed.meta);
     return hipGetLastError();
 }
 
@@ -355,12 +411,17 @@ hipError_t launch_ffn(const m26s_b1_layer* L, const Launch& k, const uint8_t* x,
 // nothing but its kernels on the stream: every event is one more packet the GPU's front end works through between two kernels.
 int enqueue(const m26s_b1_layer* L, m26s_b1_scratch* S, bool host_io, bool timed, const uint8_t* x, size_t xp, const uint8_t* xs,
             size_t xsp, const int32_t* ids, const float* w, uint32_t rows, uint16_t* bf16_out, float* partial, Outcome& out) {
-    const Shape shape{rows, L->lay.inter, S->taps, host_io, !L->all_normal};
-    if (const int rc = fit_slab(S, carve(nullptr, shape).total, out)) return rc;
-    S->last = carve(S->slab, shape);
+    if (const int rc = ready_workspace(S, shape_of(L, S, rows, host_io), out)) return rc;
     S->last_rows = rows;
-    const Launch k{S->stream, fixed_at(S->fixed), S->last, S->taps, timed ? S->planned : nullptr, timed ? S->fc1_done : nullptr,
-                   timed ? S->fc2_done : nullptr};
+    if (S->guards) {
+        ZoneTable t{};
+        t.zones = S->last.zones;
+        std::memcpy(t.zone, S->last.zone, sizeof t.zone);
+        fill_zones_kernel<<<kMaxZones, 256, 0, S->stream>>>(S->slab, t);
+        M26G_TRY(out, hipGetLastError(), "b1 red zones");
+    }
+    const Launch k{S->stream, fixed_at(S->fixed), S->last, S->taps, S->y_bf16, timed ? S->planned : nullptr,
+                   timed ? S->fc1_done : nullptr, timed ? S->fc2_done : nullptr};
     if (host_io) {  // the inputs were staged into the slab by the caller of this function
         x = S->last.x, xp = kHidden, xs = S->last.xs, xsp = kHidden / 32, ids = S->last.ids, w = S->last.weights;
         bf16_out = S->last.bf16;
@@ -436,7 +497,18 @@ static __device__ __align__(256) uint8_t scratch[kStaticBytes];
 
 namespace {
 constexpr int kStaticDevices = 64;
-uint8_t* static_base[kStaticDevices];  // the array's device address per GPU (the symbol itself is no address on the host)
+// The array's device address per GPU (the symbol itself is no address on the host). Threads that race on a
+// GPU's first call look the same address up and store the same value.
+std::atomic<uint8_t*> static_base[kStaticDevices];
+// First kernel of every call on the static workspace: the count and fault words start from zero and the 256
+// unit scale bytes are written again, so the array needs no one-time initialisation that a graph capture could
+// swallow or another stream could overtake. The zero row is never written: the array starts as zeros when the
+// code object is loaded.
+__global__ void static_begin_kernel(uint8_t* base) {
+    const Fixed f = fixed_at(base);
+    if (threadIdx.x < kMetaWords) f.meta[threadIdx.x] = threadIdx.x == kQuantWhere ? 0xffffffffu : 0u;
+    reinterpret_cast<uint32_t*>(f.unit_scales)[threadIdx.x] = 0x7f7f7f7fu;
+}
 __global__ void status_copy_kernel(uint32_t* __restrict__ out, const uint32_t* __restrict__ meta) {
     if (threadIdx.x < kMetaWords) out[threadIdx.x] = meta[threadIdx.x];
 }
@@ -509,9 +581,8 @@ int m26s_b1_ffn(const m26s_b1_layer* L, m26s_b1_scratch* S, const uint8_t* paylo
         return out.fail(1, "b1 ffn: bad rows/handles/pitch");
     const auto t0 = Clock::now();
     // Stage the caller's host arrays into the slab: rows packed to 4096 / 128 bytes, ids and weights as they are.
-    const Shape shape{rows, L->lay.inter, S->taps, true, !L->all_normal};
-    if (const int rc = fit_slab(S, carve(nullptr, shape).total, out)) return rc;
-    const Workspace ws = carve(S->slab, shape);
+    if (const int rc = ready_workspace(S, shape_of(L, S, rows, true), out)) return rc;
+    const Workspace ws = S->last;
     const size_t routes = size_t(rows) * kTopk, out_bytes = size_t(rows) * kHidden * 2;
     // The reference's daemon hands over page-locked arrays (its registered receive ring and send slot) and those
     // are copied from and to directly. Pageable arrays go through a page-locked bounce buffer of the scratch:
@@ -620,7 +691,7 @@ int m26s_b1_plan_dev(const int32_t* ids_dev, const float* weights_dev, uint32_t 
     hipError_t e = hipMemset(work, 0, 256);
     if (e == hipSuccess) {
         const PlanView pv{inverse_dev, original_routes_dev, grouped_weights_dev, static_cast<Group*>(groups_dev),
-                          reinterpret_cast<Chunk*>(work + 256), reinterpret_cast<uint32_t*>(work)};
+                          reinterpret_cast<Chunk*>(work + 256), reinterpret_cast<uint32_t*>(work), nullptr};
         plan_kernel<<<1, kPlanThreads, uint64_t(rows) * kTopk, 0>>>(ids_dev, weights_dev, rows, resident_dev, pv, 1,
                                                                      capacity * kTopk, true);
         e = hipGetLastError();
@@ -654,8 +725,8 @@ int m26s_b1_reduce_dev(const float* y_dev, const float* weights_dev, uint32_t ro
     M26G_TRY(out, hipMemset(fault_dev, 0, 4), "b1 reduce fault clear");
     if (!rows) return 0;
     const uint64_t n4 = uint64_t(rows) * (kHidden / 4);
-    reduce_kernel<<<uint32_t(n4 / 256 < 65536 ? (n4 + 255) / 256 : 65536), 256>>>(y_dev, weights_dev, rows, partial_dev,
-                                                                                bf16_dev, fault_dev, nullptr);
+    reduce_kernel<false><<<uint32_t(n4 / 256 < 65536 ? (n4 + 255) / 256 : 65536), 256>>>(y_dev, weights_dev, rows, partial_dev,
+                                                                                       bf16_dev, fault_dev, nullptr);
     M26G_TRY(out, hipGetLastError(), "b1 reduce launch");
     M26G_TRY(out, hipDeviceSynchronize(), "b1 reduce sync");
     return 0;
@@ -671,25 +742,22 @@ int m26s_b1_ffn_static(const m26s_b1_layer* L, const uint8_t* payload_dev, size_
         return out.fail(1, "b1 ffn: bad rows/handles/pitch");
     if (rows > kStaticRows)
         return out.fail(1, "b1 ffn static: %u rows exceed the %u rows the fixed workspace holds", rows, kStaticRows);
-    const Shape shape{rows, L->lay.inter, false, false, !L->all_normal};
+    const Shape shape{rows, L->lay.inter, false, false, !L->all_normal, L->all_normal, false, false};
     if (carve(nullptr, shape).total + kFixedBytes > kStaticBytes)
         return out.fail(1, "b1 ffn static: the call needs more than the fixed workspace of %zu bytes", kStaticBytes);
     const hipStream_t stream = static_cast<hipStream_t>(hip_stream);
     int device = -1;
     M26G_TRY(out, hipGetDevice(&device), "b1 ffn static device");
     if (device < 0 || device >= kStaticDevices) return out.fail(1, "b1 ffn static: device %d is beyond the %d this entry keeps track of", device, kStaticDevices);
-    if (!static_base[device]) {  // first call on this GPU: find this GPU's copy of the array and write its constants
-        uint8_t* base = nullptr;
+    uint8_t* base = static_base[device].load(std::memory_order_acquire);
+    if (!base) {  // first call on this GPU: find this GPU's copy of the array (a host-side look-up, nothing is enqueued)
         M26G_TRY(out, hipGetSymbolAddress(reinterpret_cast<void**>(&base), HIP_SYMBOL(scratch)), "b1 ffn static workspace address");
         if (!base) return out.fail(2, "b1 ffn static workspace address: null");
-        fixed_init_kernel<<<1, 256, 0, stream>>>(base);
-        M26G_TRY(out, hipGetLastError(), "b1 ffn static workspace init");
-        static_base[device] = base;
+        static_base[device].store(base, std::memory_order_release);
     }
-    uint8_t* const base = static_base[device];
-    const Launch k{stream, fixed_at(base), carve(base + kFixedBytes, shape), false, nullptr, nullptr, nullptr};
+    const Launch k{stream, fixed_at(base), carve(base + kFixedBytes, shape), false, false, nullptr, nullptr, nullptr};
     // The array keeps what the last call left: the count and fault words start every call from zero.
-    meta_reset_kernel<<<1, 64, 0, stream>>>(k.fixed.meta);
+    static_begin_kernel<<<1, 64, 0, stream>>>(base);
     M26G_TRY(out, hipGetLastError(), "b1 ffn static reset");
     M26G_TRY(out, launch_ffn(L, k, payload_dev, payload_pitch, scales_dev, scales_pitch, ids_dev, weights_dev, rows, bf16_out_dev, nullptr),
              "b1 ffn static launch");
@@ -701,6 +769,50 @@ int m26s_b1_ffn_static(const m26s_b1_layer* L, const uint8_t* payload_dev, size_
 }
 
 void m26s_b1_scratch_set_taps(m26s_b1_scratch* S, int on) { if (S) S->taps = on != 0; }
+
+int m26s_b1_scratch_set_option(m26s_b1_scratch* S, int option, int value) {
+    if (!S) return 1;
+    const bool on = value != 0;
+    switch (option) {
+    case M26S_B1_OPT_TAPS: S->taps = on; return 0;
+    case M26S_B1_OPT_SEPARATE_COMBINE: S->separate_combine = on; return 0;
+    case M26S_B1_OPT_BF16_ROUTE_ROWS: S->y_bf16 = on; return 0;
+    case M26S_B1_OPT_GUARDS:
+        if (S->guards != on) {  // the layout changes: the next call starts on a fresh slab, armed again
+            if (hipStreamSynchronize(S->stream) != hipSuccess) return 2;
+            if (S->slab) (void)hipFree(S->slab);
+            S->slab = nullptr;
+            S->slab_bytes = 0;
+            S->last = Workspace{};
+            S->guards = on;
+        }
+        return 0;
+    default: return 1;
+    }
+}
+
+int m26s_b1_scratch_check_guards(m26s_b1_scratch* S, char* err, size_t errlen) {
+    Outcome out(err, errlen);
+    if (!S || !S->guards || !S->slab || !S->last.zones) return out.fail(1, "b1 guards: not enabled, or no call made yet");
+    M26G_TRY(out, hipStreamSynchronize(S->stream), "b1 guards sync");
+    std::vector<uint8_t> host;
+    for (int i = 0; i < S->last.zones; ++i) {
+        const Zone z = S->last.zone[i];
+        host.assign(z.bytes, 0);
+        M26G_TRY(out, hipMemcpy(host.data(), S->slab + z.at, z.bytes, hipMemcpyDeviceToHost), "b1 guards download");
+        for (uint64_t b = 0; b < z.bytes; ++b)
+            if (host[b] != kGuardByte)
+                return out.fail(4, "b1 guards: red zone %d damaged at slab offset %llu (byte %llu of %llu holds 0x%02x)", i,
+                                static_cast<unsigned long long>(z.at + b), static_cast<unsigned long long>(b),
+                                static_cast<unsigned long long>(z.bytes), host[b]);
+    }
+    return 0;
+}
+
+int m26s_b1_device_memory(size_t* free_bytes, size_t* total_bytes) {
+    if (!free_bytes || !total_bytes) return 1;
+    return hipMemGetInfo(free_bytes, total_bytes) == hipSuccess ? 0 : 2;
+}
 
 int m26s_b1_scratch_view(const m26s_b1_scratch* S, int which, void** dev_ptr, size_t* bytes) {
     if (!S || !dev_ptr || !bytes || !S->slab) return 1;

@@ -188,7 +188,8 @@ __global__ void __launch_bounds__(kConformColumns) fc2_conform_kernel(Fc2Args a)
         if (r >= rows) continue;
         const int32_t route = a.plan.original[base + r];
         if (route < 0 || uint32_t(route) >= a.routes) { lost = true; continue; }
-        a.y[size_t(route) * kHidden + n] = float(acc[r]);
+        if (a.y_bf16) reinterpret_cast<uint16_t*>(a.y)[size_t(route) * kHidden + n] = uint16_t(bf16_bits_rne(float(acc[r])));
+        else a.y[size_t(route) * kHidden + n] = float(acc[r]);
     }
     if (lost) atomicOr(&meta[kFc2Fault], 5u);
 }

@@ -20,6 +20,7 @@ namespace m26g {
 typedef int v8i __attribute__((ext_vector_type(8)));
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef float v4f __attribute__((ext_vector_type(4)));
+typedef uint32_t v2u __attribute__((ext_vector_type(2)));
 
 struct Canonical {
     const uint8_t* pool[4];  // ranks x (256 quarter-slice images)
@@ -33,6 +34,7 @@ struct PlanView {
     Group* groups;
     Chunk* chunks;
     uint32_t* meta;
+    uint32_t* done;  // [rows][64] completion counts of the fused combine (see combine_completed), or null
 };
 
 // ---------------------------------------------------------------------------------------------
@@ -98,6 +100,7 @@ __global__ void __launch_bounds__(256) prepare_kernel(Canonical c, uint8_t* __re
 // expert, and the second walk places routes. Dynamic LDS holds one id byte per route.
 // ---------------------------------------------------------------------------------------------
 constexpr uint32_t kPlanThreads = 1024, kPlanWaves = kPlanThreads / 64;
+constexpr uint32_t kDoneBlocks = kHidden / 64;  // completion counts per token: one per 64 output columns
 
 __device__ __forceinline__ uint64_t same_expert_lanes(uint32_t e, bool valid) {
     uint64_t m = __ballot(valid);
@@ -149,6 +152,8 @@ plan_kernel(const int32_t* __restrict__ ids, const float* __restrict__ w, uint32
 
     for (uint32_t i = tid; i < kPlanWaves * 256; i += kPlanThreads) (&hist[0][0])[i] = 0;
     if (tid == 0) first_bad = 0xffffffffu;
+    if (p.done)  // every call starts its completion counts from zero, whatever the call before left
+        for (uint32_t i = tid; i < rows * kDoneBlocks; i += kPlanThreads) p.done[i] = 0;
     __syncthreads();
     // Validation keys order faults as the serial planner meets them: (route + 1) << 4 | check,
     // check 1 = id or residency, 2 = weight, 3 = expert repeated inside the token.
@@ -326,13 +331,16 @@ __host__ __device__ constexpr uint64_t wide_plan_words(uint32_t routes) {
 
 __global__ void __launch_bounds__(kPlanThreads)
 plan_count_kernel(const int32_t* __restrict__ ids, const float* __restrict__ w, uint32_t rows,
-                  const uint8_t* __restrict__ resident, uint32_t* __restrict__ work) {
+                  const uint8_t* __restrict__ resident, uint32_t* __restrict__ work, uint32_t* __restrict__ done) {
     __shared__ __align__(16) uint8_t id_byte[kWideRoutesPerGroup];
     __shared__ uint32_t hist[kPlanWaves][256];
     __shared__ uint8_t present[256];
     const uint32_t tid = threadIdx.x, lane = tid & 63, wv = tid >> 6, routes = rows * kTopk;
     const uint32_t first_route = blockIdx.x * kWideRoutesPerGroup;
     for (uint32_t i = tid; i < kPlanWaves * 256; i += kPlanThreads) (&hist[0][0])[i] = 0;
+    if (done)  // the completion counts of this workgroup's tokens start from zero
+        for (uint32_t i = first_route / kTopk * kDoneBlocks + tid; i < (first_route + kWideRoutesPerGroup) / kTopk * kDoneBlocks && i < rows * kDoneBlocks; i += kPlanThreads)
+            done[i] = 0;
     if (tid < 256) {
         const uint8_t here = resident[tid];
         if (here > 1 && blockIdx.x == 0) atomicMin(&work[0], 1u);
@@ -869,29 +877,178 @@ struct Fc2Args {
     const uint8_t* dqs;
     const uint8_t* zero_row;
     const uint8_t* unit_scales;
-    float* y;         // [routes][4096], original (token, slot) order, unweighted
+    float* y;         // [routes][4096], original (token, slot) order, unweighted; BF16 bits when y_bf16
     uint32_t routes;
     const uint8_t* dg;  // tile schedule only: the intermediate's scales in MFMA lane order (see Fc1Args)
     const int32_t* yrows;  // tile schedule only, [chunk][8 tiles][16]: the route (row of y) of each row, -1 for none
     const uint32_t* rowbad;  // tile schedule only: as in Fc1Args (bit 8+t: tile t holds a token in that row)
     unsigned long long* clock;  // tile schedule only, may be null: see TileClock in b1_tile.h
+    // The combine, done here by whichever wave completes a token's eighth row (plan.done != null):
+    const float* w;     // [rows][8] router weights, the caller's array
+    uint16_t* bf16;     // [rows][4096] BF16 bits out
+    float* partial;     // [rows][4096] FP32 sums out, or null
+    bool y_bf16;        // per-route rows are kept as BF16 bits (the opt-in mode of b1_serve.cu:98-143,400-405), not FP32
 };
 
-// FC2 epilogue of one wave: unweighted FP32 rows back to y[original route].
+// ---------------------------------------------------------------------------------------------
+// Stage 4b, the combine's arithmetic (kernels/b1/route_reduce.cu:61-74): per column v = 0; for slot 0..7:
+// v = RN(v + RN(w * z)), multiply and add rounded separately; BF16 RNE; a weight outside [0, FLT_MAX], a
+// nonfinite z or running sum, or a BF16 exponent of all ones fails the element group (NaN / zero out).
+// Four columns of one token. Returns false when the group failed.
+// ---------------------------------------------------------------------------------------------
+__device__ __forceinline__ bool combine4(const v4f (&z)[8], const float (&wt)[8], float (&v)[4], uint32_t (&code)[4]) {
+    bool ok = true;
+    v[0] = v[1] = v[2] = v[3] = 0.0f;
+#pragma unroll
+    for (int s = 0; s < 8; ++s) {
+        ok = ok && wt[s] >= 0.0f && wt[s] <= FLT_MAX;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            ok = ok && fabsf(z[s][k]) <= FLT_MAX;
+            v[k] = __fadd_rn(v[k], __fmul_rn(wt[s], z[s][k]));
+            ok = ok && fabsf(v[k]) <= FLT_MAX;
+        }
+    }
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        const uint32_t b = __float_as_uint(v[k]);
+        code[k] = (b + 0x7fffu + ((b >> 16) & 1u)) >> 16;
+        ok = ok && (code[k] & 0x7f80u) != 0x7f80u;
+    }
+    if (!ok) {
+        v[0] = v[1] = v[2] = v[3] = __uint_as_float(0x7fc00000u);
+        code[0] = code[1] = code[2] = code[3] = 0;
+    }
+    return ok;
+}
+// BF16 bits -> binary32, and the reference's store rule for BF16 per-route rows (connected.cu:41-44).
+__device__ __forceinline__ float bf16_value(uint32_t bits16) { return __uint_as_float(bits16 << 16); }
+__device__ __forceinline__ uint32_t bf16_bits_rne(float v) {
+    const uint32_t b = __float_as_uint(v);
+    return (b + 0x7fffu + ((b >> 16) & 1u)) >> 16;
+}
+
+// Hand-over of per-route rows between waves of one launch that run on different XCDs, each with an L2 of
+// its own: the rows are stored with device-scope write-through stores (sc1) and read back with device-scope
+// loads (sc1), which no L2 answers from a stale line; between them stand the writer's wait for its stores'
+// acknowledgements and a device-scope atomic on the token's count. The language-level fence that would
+// order plain stores instead writes the whole L2 back (27 times the time of this form in a probe of 65,536
+// rows of 2 KB, which also showed 1.8 million stale values per launch with plain stores and none with sc1).
+// The stores are asm statements, and with them comes a duty the compiler otherwise carries: a store of more
+// than eight bytes reads the upper half of its data a little after it issues, so the next two wait states
+// must not write those registers. The compiler cannot see that an asm statement is such a store (it reused
+// the registers at once, and the last two of four columns came out wrong now and then): the wait states are
+// part of the statement.
+__device__ __forceinline__ void store_route4(const Fc2Args& a, uint32_t route, uint32_t col, const v4f v) {
+    if (a.y_bf16) {
+        uint16_t* dst = reinterpret_cast<uint16_t*>(a.y) + size_t(route) * kHidden + col;
+        const v2u packed = {bf16_bits_rne(v.x) | bf16_bits_rne(v.y) << 16, bf16_bits_rne(v.z) | bf16_bits_rne(v.w) << 16};
+        asm volatile("global_store_dwordx2 %0, %1, off sc1\n\ts_nop 1" ::"v"(dst), "v"(packed) : "memory");
+    } else {
+        float* dst = a.y + size_t(route) * kHidden + col;
+        asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 1" ::"v"(dst), "v"(v) : "memory");
+    }
+}
+__device__ __forceinline__ void wait_stores_acknowledged() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+
+// One more row of `token` lies complete in y for output block ob (64 columns): returns true for the lane
+// whose row was the token's eighth. Integer atomics decide only who sums, never the order of the sum.
+__device__ __forceinline__ bool completes_token(const Fc2Args& a, uint32_t token, uint32_t ob) {
+    return __hip_atomic_fetch_add(a.plan.done + size_t(token) * kDoneBlocks + ob, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == kTopk - 1;
+}
+
+// The wave sums, for output block ob, every token a lane names in `token` (-1: none): sixteen lanes and four
+// columns each per token, four tokens at a time, the eight rows of a token fetched before the first is used,
+// summed in slot order exactly as reduce_kernel does.
+__device__ __forceinline__ void combine_completed(const Fc2Args& a, uint32_t ob, uint32_t lane, int32_t token) {
+    uint64_t todo = __ballot(token >= 0);
+    bool failed = false;
+    while (todo) {
+        uint32_t from = 64;  // the lane that names this lane group's token
+#pragma unroll
+        for (uint32_t i = 0; i < 4; ++i) {
+            const uint32_t first = todo ? uint32_t(__builtin_ctzll(todo)) : 64u;
+            if (i == (lane >> 4)) from = first;
+            todo &= todo - 1;
+        }
+        const int32_t mine = __shfl(token, int(from & 63u));
+        if (from < 64) {
+            const uint32_t col = ob * 64 + 4 * (lane & 15);
+            const size_t first_row = size_t(mine) * kTopk;
+            v4f z[8];
+            float wt[8];
+            if (a.y_bf16) {
+                const uint16_t* src = reinterpret_cast<const uint16_t*>(a.y) + first_row * kHidden + col;
+                v2u raw[8];
+                asm volatile(
+                    "global_load_dwordx2 %0, %8, off sc1\n\tglobal_load_dwordx2 %1, %9, off sc1\n\t"
+                    "global_load_dwordx2 %2, %10, off sc1\n\tglobal_load_dwordx2 %3, %11, off sc1\n\t"
+                    "global_load_dwordx2 %4, %12, off sc1\n\tglobal_load_dwordx2 %5, %13, off sc1\n\t"
+                    "global_load_dwordx2 %6, %14, off sc1\n\tglobal_load_dwordx2 %7, %15, off sc1\n\t"
+                    "s_waitcnt vmcnt(0)"
+                    : "=&v"(raw[0]), "=&v"(raw[1]), "=&v"(raw[2]), "=&v"(raw[3]), "=&v"(raw[4]), "=&v"(raw[5]), "=&v"(raw[6]), "=&v"(raw[7])
+                    : "v"(src), "v"(src + kHidden), "v"(src + 2 * kHidden), "v"(src + 3 * kHidden), "v"(src + 4 * kHidden),
+                      "v"(src + 5 * kHidden), "v"(src + 6 * kHidden), "v"(src + 7 * kHidden)
+                    : "memory");
+#pragma unroll
+                for (int s = 0; s < 8; ++s)
+                    z[s] = v4f{bf16_value(raw[s].x & 0xffffu), bf16_value(raw[s].x >> 16), bf16_value(raw[s].y & 0xffffu), bf16_value(raw[s].y >> 16)};
+            } else {
+                const float* src = a.y + first_row * kHidden + col;
+                asm volatile(
+                    "global_load_dwordx4 %0, %8, off sc1\n\tglobal_load_dwordx4 %1, %9, off sc1\n\t"
+                    "global_load_dwordx4 %2, %10, off sc1\n\tglobal_load_dwordx4 %3, %11, off sc1\n\t"
+                    "global_load_dwordx4 %4, %12, off sc1\n\tglobal_load_dwordx4 %5, %13, off sc1\n\t"
+                    "global_load_dwordx4 %6, %14, off sc1\n\tglobal_load_dwordx4 %7, %15, off sc1\n\t"
+                    "s_waitcnt vmcnt(0)"
+                    : "=&v"(z[0]), "=&v"(z[1]), "=&v"(z[2]), "=&v"(z[3]), "=&v"(z[4]), "=&v"(z[5]), "=&v"(z[6]), "=&v"(z[7])
+                    : "v"(src), "v"(src + kHidden), "v"(src + 2 * kHidden), "v"(src + 3 * kHidden), "v"(src + 4 * kHidden),
+                      "v"(src + 5 * kHidden), "v"(src + 6 * kHidden), "v"(src + 7 * kHidden)
+                    : "memory");
+            }
+#pragma unroll
+            for (int s = 0; s < 8; ++s) wt[s] = a.w[first_row + s];
+            float v[4];
+            uint32_t code[4];
+            failed = !combine4(z, wt, v, code) || failed;
+            if (a.partial) *reinterpret_cast<v4f*>(a.partial + size_t(mine) * kHidden + col) = v4f{v[0], v[1], v[2], v[3]};
+            *reinterpret_cast<uint2*>(a.bf16 + size_t(mine) * kHidden + col) = make_uint2(code[0] | (code[1] << 16), code[2] | (code[3] << 16));
+        }
+    }
+    if (failed) atomicOr(&a.plan.meta[kReduceFault], 8u);  // Status::nonfinite
+}
+
+// FC2 epilogue of one wave: unweighted rows back to y[original route]; then, with the combine fused, one count
+// per row and the sum of every token this wave's rows completed.
 template <int TT>
 __device__ __forceinline__ void fc2_finish(const Fc2Args& a, uint32_t ob, uint32_t lane, v4f (&acc)[4][TT],
                                            const int32_t (&route)[TT]) {
     const uint32_t g = lane >> 4;
     bool lost = false;
+    // The stores below are asm statements (they carry a cache policy the language has no word for), and the
+    // compiler's hazard tables do not look inside one: a matrix instruction's result lands up to eight passes
+    // after issue, and a store issued sooner sends what the register held before (seen as the last two of four
+    // columns of a tile's rows 12..15 wrong, now and then). These statements take every accumulator as an operand,
+    // so they sit behind the last MFMA, and spend the wait states the compiler would have inserted.
+#pragma unroll
+    for (int tt = 0; tt < TT; ++tt)
+        asm volatile("s_nop 15\n\ts_nop 15" : "+v"(acc[0][tt]), "+v"(acc[1][tt]), "+v"(acc[2][tt]), "+v"(acc[3][tt]));
 #pragma unroll
     for (int tt = 0; tt < TT; ++tt) {
         if (route[tt] < 0) continue;
         if (uint32_t(route[tt]) >= a.routes) { lost = true; continue; }
-        float* dst = a.y + size_t(route[tt]) * kHidden + ob * 64 + 4 * g;
 #pragma unroll
-        for (int t = 0; t < 4; ++t) *reinterpret_cast<v4f*>(dst + 16 * t) = acc[t][tt];
+        for (int t = 0; t < 4; ++t) store_route4(a, uint32_t(route[tt]), ob * 64 + 16 * t + 4 * g, acc[t][tt]);
     }
     if (lost) atomicOr(&a.plan.meta[kFc2Fault], 5u);
+    if (!a.plan.done) return;
+    wait_stores_acknowledged();
+#pragma unroll
+    for (int tt = 0; tt < TT; ++tt) {  // lanes 0..15 hold one row each of the tile (the other lane groups hold the same rows)
+        const bool counts = g == 0 && route[tt] >= 0 && uint32_t(route[tt]) < a.routes;
+        const int32_t token = counts && completes_token(a, uint32_t(route[tt]) >> 3, ob) ? route[tt] >> 3 : -1;
+        combine_completed(a, ob, lane, token);
+    }
 }
 
 // One wave's share of FC2 for a chunk of TT groups: 64 output columns x 16*TT rows.
@@ -944,10 +1101,12 @@ __global__ void __launch_bounds__(256) fc2_kernel(Fc2Args a) {
     else fc2_body<(NT >= 8 ? 8 : 1)>(a, ch, ob, lane);
 }
 
-// Stage 4b: router-weighted combine. Per (token, column): v = 0; for slot 0..7:
-// v = RN(v + RN(w * z)) with two roundings; BF16 RNE; nonfinite or negative inputs, a nonfinite
-// running sum or a BF16 exponent of all ones raise the fault word. Four columns per thread.
-__global__ void __launch_bounds__(256) reduce_kernel(const float* __restrict__ y, const float* __restrict__ w,
+// Stage 4b as a launch of its own (the conforming arm, and the stand-alone entry): the same arithmetic
+// (combine4). Four columns per thread. Y16: the per-route rows are BF16 bits (crates/mimo26-spark/kernels/
+// b1_serve.cu:98-143: same order, same roundings and fault rules on the widened values, no FP32 sum kept
+// by the reference; here `partial` is still written when asked for).
+template <bool Y16>
+__global__ void __launch_bounds__(256) reduce_kernel(const void* __restrict__ y_rows, const float* __restrict__ w,
                                                      uint32_t rows, float* __restrict__ partial,
                                                      uint16_t* __restrict__ bf16, uint32_t* __restrict__ fault,
                                                      const uint32_t* __restrict__ gate) {
@@ -957,34 +1116,25 @@ __global__ void __launch_bounds__(256) reduce_kernel(const float* __restrict__ y
     for (uint64_t i = uint64_t(blockIdx.x) * blockDim.x + threadIdx.x; i < n4; i += uint64_t(gridDim.x) * blockDim.x) {
         const uint64_t row = i / (kHidden / 4), col = (i % (kHidden / 4)) * 4;
         v4f z[8];
+        if (Y16) {
+            const uint16_t* y = static_cast<const uint16_t*>(y_rows);
 #pragma unroll
-        for (int s = 0; s < 8; ++s)  // read once: streamed past the caches (6.3 against 4.9 TB/s at 8192 rows)
-            z[s] = __builtin_nontemporal_load(reinterpret_cast<const v4f*>(y + (row * 8 + s) * kHidden + col));
-        float v[4] = {0.f, 0.f, 0.f, 0.f};
-        bool ok = true;
-#pragma unroll
-        for (int s = 0; s < 8; ++s) {
-            const float wt = w[row * 8 + s];
-            ok = ok && wt >= 0.0f && wt <= FLT_MAX;
-#pragma unroll
-            for (int k = 0; k < 4; ++k) {
-                ok = ok && fabsf(z[s][k]) <= FLT_MAX;
-                v[k] = __fadd_rn(v[k], __fmul_rn(wt, z[s][k]));
-                ok = ok && fabsf(v[k]) <= FLT_MAX;
+            for (int s = 0; s < 8; ++s) {
+                const v2u raw = __builtin_nontemporal_load(reinterpret_cast<const v2u*>(y + (row * 8 + s) * kHidden + col));
+                z[s] = v4f{bf16_value(raw.x & 0xffffu), bf16_value(raw.x >> 16), bf16_value(raw.y & 0xffffu), bf16_value(raw.y >> 16)};
             }
-        }
-        uint32_t code[4];
+        } else {
+            const float* y = static_cast<const float*>(y_rows);
 #pragma unroll
-        for (int k = 0; k < 4; ++k) {
-            const uint32_t b = __float_as_uint(v[k]);
-            code[k] = (b + 0x7fffu + ((b >> 16) & 1u)) >> 16;
-            ok = ok && (code[k] & 0x7f80u) != 0x7f80u;
+            for (int s = 0; s < 8; ++s)  // read once: streamed past the caches (6.3 against 4.9 TB/s at 8192 rows)
+                z[s] = __builtin_nontemporal_load(reinterpret_cast<const v4f*>(y + (row * 8 + s) * kHidden + col));
         }
-        if (!ok) {
-            failed = true;
-            v[0] = v[1] = v[2] = v[3] = __uint_as_float(0x7fc00000u);
-            code[0] = code[1] = code[2] = code[3] = 0;
-        }
+        float wt[8];
+#pragma unroll
+        for (int s = 0; s < 8; ++s) wt[s] = w[row * 8 + s];
+        float v[4];
+        uint32_t code[4];
+        failed = !combine4(z, wt, v, code) || failed;
         if (partial) *reinterpret_cast<v4f*>(partial + row * kHidden + col) = v4f{v[0], v[1], v[2], v[3]};
         *reinterpret_cast<uint2*>(bf16 + row * kHidden + col) = make_uint2(code[0] | (code[1] << 16), code[2] | (code[3] << 16));
     }

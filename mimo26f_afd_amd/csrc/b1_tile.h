@@ -473,10 +473,21 @@ __device__ __forceinline__ void fc2_tile_body(const Fc2Args& a, const Chunk ch, 
             const int32_t rt = route[tt][j];
             if (rt < 0) continue;
             if (uint32_t(rt) >= a.routes) { lost = true; continue; }
-            *reinterpret_cast<v4f*>(a.y + size_t(rt) * kHidden + ob * 64 + cell * 4) = v;
+            store_route4(a, uint32_t(rt), ob * 64 + cell * 4, v);
         }
     }
     if (lost) atomicOr(&a.plan.meta[kFc2Fault], 5u);
+    if (!a.plan.done) return;
+    // The combine, fused: one count per row this wave has just written, then the sum of every token whose eighth
+    // row that was (b1_kernels.h, combine_completed). A lane takes rows lane and lane + 64 of the chunk.
+    wait_stores_acknowledged();
+#pragma unroll 1
+    for (int half = 0; half < TT / 4; ++half) {
+        const int32_t rt = a.yrows[c * 128 + half * 64 + lane2];
+        const bool counts = rt >= 0 && uint32_t(rt) < a.routes;
+        const int32_t token = counts && completes_token(a, uint32_t(rt) >> 3, ob) ? rt >> 3 : -1;
+        combine_completed(a, ob, lane2, token);
+    }
 }
 
 // The clock a tile launch ran at. The shader clock of these parts is not a constant of the launch: under the

@@ -20,6 +20,10 @@
  *   orc_reduce          - the compiled reference reduce_host where it builds, committed
  *                         vectors, and the reference's closed-form order / non-fused /
  *                         subnormal / BF16-midpoint vectors.
+ *   orc_reduce_bf16y,
+ *   orc_bf16_store_rows - identity with orc_reduce on the widened rows (a function pinned above, other
+ *                         code), hand-worked sums with BF16 midpoints at the store and at the output, the
+ *                         order witness (a sum that differs in any other slot order) and the fault cases.
  *   orc_silu_up         - the reference's four retained (g,u)->h witnesses and specials.
  *   orc_expert_ffn,
  *   orc_layer_ffn       - composition of the above; closed-form synthetic projections with
@@ -311,6 +315,34 @@ uint32_t orc_reduce(const float* y, const float* w, size_t rows, size_t cols, fl
             if (bf16) bf16[t * cols + c] = code;
         }
     return ORC_OK;
+}
+
+/* The opt-in BF16 per-route mode (MIMO26_B1_Y=bf16). FC2's store rule, crates/mimo26-expert/kernels/b1/
+ * connected.cu:41-44: BF16 bits by the integer round-to-nearest-even, no special cases. */
+void orc_bf16_store_rows(const float* y, size_t n, uint16_t* out) {
+    for (size_t i = 0; i < n; ++i) out[i] = orc_bf16_rne(y[i]);
+}
+
+/* crates/mimo26-spark/kernels/b1_serve.cu:98-143 (reduce_bf16y): route_reduce's sum on the widened BF16
+ * rows, same slot order, separately rounded multiply and add, same finite / sign rules, BF16 RNE out, no
+ * FP32 sum kept. Returns 0, or 5 (the value that kernel's fault word takes) at the first violating element. */
+uint32_t orc_reduce_bf16y(const uint16_t* y16, const float* w, size_t rows, size_t cols, uint16_t* bf16) {
+    for (size_t t = 0; t < rows; ++t)
+        for (size_t c = 0; c < cols; ++c) {
+            volatile float v = 0.0f;
+            for (int s = 0; s < 8; ++s) {
+                const float wt = w[t * 8 + s], z = bits_f32((uint32_t)y16[(t * 8 + s) * cols + c] << 16);
+                if (!(wt >= 0.0f && wt <= FLT_MAX) || !(z >= -FLT_MAX && z <= FLT_MAX)) return 5;
+                volatile float p = wt * z;
+                v = v + p;
+                if (!(v >= -FLT_MAX && v <= FLT_MAX)) return 5;
+            }
+            const uint32_t b = f32_bits(v);
+            const uint16_t code = (uint16_t)((b + 0x7fffu + ((b >> 16) & 1u)) >> 16);
+            if ((code & 0x7f80u) == 0x7f80u) return 5;
+            bf16[t * cols + c] = code;
+        }
+    return 0;
 }
 
 /* ------------------------------------------------------------------------------------------

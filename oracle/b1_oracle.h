@@ -82,6 +82,11 @@ float orc_silu_up(float gate, float up);
 uint32_t orc_reduce(const float* y, const float* w, size_t rows, size_t cols, float* partial,
                     uint16_t* bf16);
 
+/* The opt-in BF16 per-route mode: FC2's store rule (FP32 -> BF16 bits, round to nearest even by the integer
+ * formula) and the combine over such rows [rows][8][cols] (no FP32 sum is kept). Returns 0 or 5. */
+void orc_bf16_store_rows(const float* y, size_t n, uint16_t* out);
+uint32_t orc_reduce_bf16y(const uint16_t* y16, const float* w, size_t rows, size_t cols, uint16_t* bf16);
+
 /* --- expert FFN ---------------------------------------------------------------------- */
 /* A layer's weights: `ranks` pools (1 = one TP4 rank's share, I = 512; 4 = all four rank
  * images, I = 2048), each 256 quarter-slice images back to back in expert-id order. */

@@ -51,6 +51,8 @@ def _load():
     lib.orc_activation_decode.restype = C.c_size_t
     lib.orc_plan.restype = C.c_uint32
     lib.orc_reduce.restype = C.c_uint32
+    lib.orc_reduce_bf16y.restype = C.c_uint32
+    lib.orc_bf16_store_rows.restype = None
     lib.orc_expert_ffn.restype = C.c_uint32
     lib.orc_layer_ffn.restype = C.c_uint32
     lib.orc_layer_ffn_efp32.restype = C.c_uint32
@@ -253,6 +255,24 @@ def reduce(y: np.ndarray, w: np.ndarray):
     return int(st), partial, bf16
 
 
+def bf16_store_rows(y: np.ndarray) -> np.ndarray:
+    """FC2's store rule of the BF16 per-route mode: FP32 -> BF16 bits (connected.cu:41-44)."""
+    y = np.ascontiguousarray(y, np.float32)
+    out = np.zeros(y.shape, np.uint16)
+    LIB.orc_bf16_store_rows(_p(y, _f32p), C.c_size_t(y.size), _p(out, _u16p))
+    return out
+
+
+def reduce_bf16y(y16: np.ndarray, w: np.ndarray):
+    """The combine over BF16 per-route rows [rows*8, cols] (b1_serve.cu:98-143): (status, bf16 [rows, cols])."""
+    y16 = np.ascontiguousarray(y16, np.uint16)
+    w = np.ascontiguousarray(w, np.float32).reshape(-1, 8)
+    rows, cols = w.shape[0], y16.shape[-1]
+    bf16 = np.zeros((rows, cols), np.uint16)
+    st = LIB.orc_reduce_bf16y(_p(y16, _u16p), _p(w, _f32p), C.c_size_t(rows), C.c_size_t(cols), _p(bf16, _u16p))
+    return int(st), bf16
+
+
 def _layer(pools) -> _Layer:
     L = _Layer()
     for i, p in enumerate(pools):
@@ -302,11 +322,18 @@ def layer_ffn(pools, x_payload, x_scales, ids, weights, threads: int = 0, want_r
 
 
 # ---- the reference's own host units, where built (differential checks only) -------------------
+_REF_PATH = os.path.join(HERE, "_ref", "libb1ref.so")
+
+
+def ref_available() -> bool:
+    """True where the reference's host units were built; asking does not load them."""
+    return os.path.exists(_REF_PATH)
+
+
 def _load_ref():
-    path = os.path.join(HERE, "_ref", "libb1ref.so")
-    if not os.path.exists(path):
+    if not ref_available():
         return None
-    lib = C.CDLL(path)
+    lib = C.CDLL(_REF_PATH)
     lib.ref_mxfp4_bits.restype = C.c_uint32
     lib.ref_mxfp4_bits.argtypes = [C.c_uint32, C.c_uint32]
     for f in (lib.ref_quant_v1, lib.ref_plan, lib.ref_reduce):
@@ -314,7 +341,17 @@ def _load_ref():
     return lib
 
 
-REF = _load_ref()
+_REF = None
+
+
+def __getattr__(name):
+    """`REF` is loaded on first use, so a process that only runs the GPU parity tests never maps it."""
+    global _REF
+    if name == "REF":
+        if _REF is None:
+            _REF = _load_ref()
+        return _REF
+    raise AttributeError(name)
 
 
 def ref_quant_v1(h: np.ndarray, fill: int = 0xA5):
@@ -323,12 +360,12 @@ def ref_quant_v1(h: np.ndarray, fill: int = 0xA5):
     payload = np.full(h.shape, fill, np.uint8)
     scales = np.full(h.shape[:-1] + (h.shape[-1] // 32,), fill, np.uint8)
     faults = np.zeros(n // 32, np.uint32)
-    st = REF.ref_quant_v1(_p(h, _f32p), C.c_uint64(n), _p(payload, _u8p), _p(scales, _u8p), _p(faults, _u32p))
+    st = __getattr__("REF").ref_quant_v1(_p(h, _f32p), C.c_uint64(n), _p(payload, _u8p), _p(scales, _u8p), _p(faults, _u32p))
     return payload, scales, faults.reshape(scales.shape), int(st)
 
 
 def ref_plan(capacity, ids, weights, resident=None, out: Plan | None = None) -> Plan:
-    return _plan_call(REF.ref_plan, capacity, ids, weights, resident, out or Plan(capacity))
+    return _plan_call(__getattr__("REF").ref_plan, capacity, ids, weights, resident, out or Plan(capacity))
 
 
 def ref_reduce(y: np.ndarray, w: np.ndarray):
@@ -338,5 +375,5 @@ def ref_reduce(y: np.ndarray, w: np.ndarray):
     partial = np.zeros((rows, HIDDEN), np.float32)
     bf16 = np.zeros((rows, HIDDEN), np.uint16)
     fault = np.zeros(1, np.uint32)
-    st = REF.ref_reduce(_p(y, _f32p), _p(w, _f32p), C.c_uint32(rows), _p(partial, _f32p), _p(bf16, _u16p), _p(fault, _u32p))
+    st = __getattr__("REF").ref_reduce(_p(y, _f32p), _p(w, _f32p), C.c_uint32(rows), _p(partial, _f32p), _p(bf16, _u16p), _p(fault, _u32p))
     return int(st), partial, bf16

@@ -160,6 +160,65 @@ def test_mfma_decodes_every_code_under_every_ordinary_scale(per_set):
         assert every <= pairs, (name, sorted(every - pairs)[:8])
 
 
+def test_swiglu_on_deeply_negative_gates():
+    """Gates between -16 and -360 fed as exact single products. Down to about -87.3 the exponential is a normal
+    binary32 number and the activation stays within the usual few ulp of the CPU rule. Below that the CPU rule's
+    exp (and the expf of the reference's kernels, crates/mimo26-expert/kernels/b1/grouped.cu:89) is a subnormal,
+    which the hardware 2^x returns as zero: the kernel's h is a signed zero where the rule's is at most
+    104 * 2^-126 |u| in magnitude, twenty orders of magnitude under the quantizer's floor, and the bytes of the
+    requantised intermediate are the same either way."""
+    pool = np.full(synth.EXPERTS * synth.IMAGE_BYTES, 0x22, np.uint8)
+    n = np.arange(512)
+    img = blank_image()
+    gate_pay, up_pay = np.zeros((512, 2048), np.uint8), np.zeros((512, 2048), np.uint8)
+    gate_pay[:, 0] = np.array([0xF, 0xE, 0xD, 0xC], np.uint8)[n % 4]          # -6, -4, -3, -2 at k = 0 ...
+    gate_sc, up_sc = np.full((512, 128), 127, np.uint8), np.full((512, 128), 127, np.uint8)
+    gate_sc[:, 0] = 127 + (n // 4) % 2                                          # ... times 1 or 2
+    up_pay[:, 0] = 0x2                                                          # +1.0 at k = 0 ...
+    up_sc[:, 0] = 127 - n % 8                                                   # ... times 2^-(n % 8)
+    img[0:gate_pay.size] = gate_pay.reshape(-1)
+    img[synth.GATE_SCALES:synth.UP_PAYLOAD] = gate_sc.reshape(-1)
+    img[synth.UP_PAYLOAD:synth.UP_PAYLOAD + up_pay.size] = up_pay.reshape(-1)
+    img[synth.UP_SCALES:synth.DOWN_PAYLOAD] = up_sc.reshape(-1)
+    pool[:synth.IMAGE_BYTES] = img
+    for e in range(1, 8):
+        pool[e * synth.IMAGE_BYTES:(e + 1) * synth.IMAGE_BYTES] = blank_image()
+    layer = DeviceLayer([pool]).layer
+    assert layer.all_scales_normal()
+    rows = 16
+    payload = np.zeros((rows, 4096), np.uint8)
+    payload[:, 0] = np.array([0x50 + i for i in range(8)] + [0x58 + i for i in range(8)], np.uint8)   # 8..15, 16..30
+    scales = np.full((rows, 128), 127, np.uint8)
+    x0 = E4M3[payload[:, 0]].astype(np.float64)
+    assert x0.tolist() == [8, 9, 10, 11, 12, 13, 14, 15, 16, 18, 20, 22, 24, 26, 28, 30]
+    ids = np.tile(np.arange(8, dtype=np.int32), (rows, 1))
+    w = np.full((rows, 8), 0.125, np.float32)
+    wl = synth.Workload("deep negative gates", -1, 0, 1, rows, ids, w, np.zeros((rows, 4096), np.float32), payload, scales)
+    scratch = b1.Scratch()
+    scratch.set_taps(True)
+    stats, _, _ = run_ffn_dev(layer, scratch, wl, want_partial=False)
+    groups = scratch.view("groups", O.GROUP_DTYPE, stats.groups)
+    gi = int(np.flatnonzero(groups["expert"] == 0)[0])
+    sl = slice(gi * 16, gi * 16 + rows)
+    taps = {k: scratch.view(k, np.float32, stats.groups * 16 * 512).reshape(-1, 512)[sl] for k in ("gate", "up", "h")}
+    mid = scratch.view("mid_payload", np.uint8, stats.groups * 16 * 512).reshape(-1, 512)[sl]
+    wg = MXFP4[gate_pay[:, 0] & 15, gate_sc[:, 0]].astype(np.float64)
+    wu = MXFP4[up_pay[:, 0] & 15, up_sc[:, 0]].astype(np.float64)
+    assert np.array_equal(taps["gate"].astype(np.float64), x0[:, None] * wg[None, :])        # exact single products
+    assert np.array_equal(taps["up"].astype(np.float64), x0[:, None] * wu[None, :])
+    g, u = taps["gate"], taps["up"]
+    assert g.min() == -360 and ((g <= -80) & (g >= -104)).sum() > 500 and ((g > -87) & (g <= -16)).sum() > 1000
+    rule = O.silu_up(g, u)
+    diff = np.abs(taps["h"].astype(np.float64) - rule.astype(np.float64))
+    normal_exp = g > -87.0                                                       # exp(g) is a normal binary32 number
+    assert np.all(diff[normal_exp] <= 8 * np.spacing(np.abs(rule[normal_exp])))
+    assert np.all(diff[~normal_exp] <= 2.0 ** -119 * np.abs(u[~normal_exp]))
+    assert np.all(np.signbit(taps["h"]))                                         # negative gate, positive up: the sign survives a flushed zero
+    qp, _, qf = O.quant_v1(rule)
+    assert not qf.any() and np.array_equal(qp[~normal_exp], mid[~normal_exp])    # the requantised bytes do not see it
+    assert np.mean(qp == mid) > 0.995
+
+
 def exceptional_pool(wl, seed):
     """A rank pool of wl's touched experts with exceptional weight scale bytes sown over all three
     projections of every touched expert: bytes 0 and 1 in about one block in 64 (decoded weights down to

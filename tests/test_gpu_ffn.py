@@ -191,13 +191,6 @@ def test_ragged_sizes_across_the_schedules(scratch):
         check_stages(scratch, layer, wl, pools, stats, experts=2)
 
 
-@pytest.fixture(scope="module")
-def full_layer():
-    wl = synth.make(2)
-    pools = wl.pools()
-    return wl, pools, DeviceLayer(pools).layer
-
-
 def test_decode_layer_full_intermediate(scratch, full_layer):
     """configs[2]: 256 experts x I 2048 on one GPU, 128 tokens, every row against the CPU reference."""
     wl, pools, layer = full_layer

@@ -14,7 +14,7 @@ import b1_oracle as O
 
 GOLD = os.path.join(os.path.dirname(__file__), "golden")
 FIX = np.load(os.path.join(GOLD, "b1_host_units.npz"))
-needs_ref = pytest.mark.skipif(O.REF is None, reason="oracle/_ref not built (reference tree absent)")
+needs_ref = pytest.mark.skipif(not O.ref_available(), reason="oracle/_ref not built (reference tree absent)")
 CODEBOOK = [0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0]
 F32MAX = float(np.finfo(np.float32).max)
 

@@ -12,7 +12,7 @@ import b1_oracle as O
 from mimo26f_afd_amd import synth
 
 FIX = np.load(os.path.join(os.path.dirname(__file__), "golden", "b1_host_units.npz"))
-needs_ref = pytest.mark.skipif(O.REF is None, reason="oracle/_ref not built (reference tree absent)")
+needs_ref = pytest.mark.skipif(not O.ref_available(), reason="oracle/_ref not built (reference tree absent)")
 
 
 # ---- planner -------------------------------------------------------------------------------------
@@ -174,6 +174,63 @@ def test_reduce_live_differential():
     w = rng.random((3, 8)).astype(np.float32)
     a, b = O.reduce(y, w), O.ref_reduce(y, w)
     assert a[0] == b[0] == 0 and np.array_equal(a[1], b[1]) and np.array_equal(a[2], b[2])
+
+
+# ---- the opt-in BF16 per-route mode (crates/mimo26-spark/kernels/b1_serve.cu:98-143, connected.cu:41-44) ----
+def _one16(z_bits, ws):
+    y = np.zeros((8, 4), np.uint16); w = np.ones((1, 8), np.float32)
+    y[:len(z_bits), 0] = z_bits
+    w[0, :len(ws)] = ws
+    return O.reduce_bf16y(y, w)
+
+
+def test_bf16_store_rule_hand_worked():
+    """FC2's store in that mode: nearest BF16, ties to even, by the integer formula (no special cases)."""
+    v = np.array([1.0, 1.0 + 2.0 ** -8, 1.0 + 3 * 2.0 ** -8, 1.0 + 2.0 ** -8 + 2.0 ** -20, -(1.0 + 2.0 ** -8), 0.0, -0.0,
+                  2.0 ** -133, 3.3895314e38, np.inf], np.float32)
+    want = [0x3F80, 0x3F80, 0x3F82, 0x3F81, 0xBF80, 0x0000, 0x8000, 0x0001, 0x7F7F, 0x7F80]
+    assert O.bf16_store_rows(v).tolist() == want
+    assert O.bf16_store_rows(np.array([3.4028235e38], np.float32))[0] == 0x7F80      # FLT_MAX rounds up into the exponent of all ones
+    rng = np.random.default_rng(4)
+    x = (rng.standard_normal(20000) * np.exp2(rng.integers(-100, 100, 20000))).astype(np.float32)
+    got = O.bf16_store_rows(x).astype(np.uint32) << 16
+    lo, hi = x.view(np.uint32) & 0xFFFF0000, (x.view(np.uint32) & 0xFFFF0000) + 0x10000   # the two neighbours on the BF16 grid
+    d_lo = np.abs(x.astype(np.float64) - lo.view(np.float32)); d_hi = np.abs(hi.view(np.float32).astype(np.float64) - x)
+    nearest = np.where(d_lo < d_hi, lo, np.where(d_hi < d_lo, hi, np.where((lo >> 16) & 1, hi, lo)))
+    assert np.array_equal(got, nearest)
+
+
+def test_reduce_bf16y_hand_worked_vectors():
+    one, big = 0x3F80, 0x4CBF                                                    # 1.0 and 1.0e8 rounded to BF16 (100139008)
+    st, b = _one16([big, one, big | 0x8000, 0x4040], [])                         # (big + 1 - big) + 3 = 3 only in slot order
+    assert st == 0 and b[0, 0] == 0x4040
+    st, b = _one16([0x3F81, 0x3F81], [0.5, 0.5])                                 # 1.0078125: exact in binary32, a BF16 midpoint at the output
+    assert st == 0 and b[0, 0] == 0x3F81
+    st, b = _one16([0x3F80, 0x3B80], [1.0, 1.0])                                 # 1 + 2^-8: tie, to even
+    assert st == 0 and b[0, 0] == 0x3F80
+    st, b = _one16([0x3F80, 0x3B80, 0x3B80, 0x3B80], [1.0, 1.0, 1.0, 1.0])       # 1 + 3 * 2^-8: tie, to even, upwards
+    assert st == 0 and b[0, 0] == 0x3F82
+    st, b = _one16([0x0080], [0.5])                                              # 2^-126 * 0.5: the subnormal product is kept
+    assert st == 0 and b[0, 0] == 0x0040
+    for bad in (np.nan, np.inf, -1.0):
+        assert _one16([one], [bad])[0] == 5
+    assert _one16([0x7F80], [])[0] == 5 and _one16([0x7FC0], [])[0] == 5 and _one16([0xFF80], [])[0] == 5
+    assert _one16([0x7F7F, 0x7F7F], [])[0] == 5                                  # running sum overflows
+    assert _one16([0x7F7F], [2.0])[0] == 5                                       # product overflows
+
+
+def test_reduce_bf16y_is_the_pinned_combine_on_widened_rows():
+    """Different code, same contract: orc_reduce (pinned by the reference's reduce_host and its vectors) on the
+    rows widened to binary32 gives the same BF16 bits."""
+    rng = np.random.default_rng(12)
+    y = (rng.standard_normal((5, 8, 512)) * np.exp2(rng.integers(-40, 40, (5, 8, 1)))).astype(np.float32)
+    w = rng.random((5, 8)).astype(np.float32)
+    y16 = O.bf16_store_rows(y)
+    wide = (y16.astype(np.uint32) << 16).view(np.float32)
+    st, _, want = O.reduce(wide, w)
+    st16, got = O.reduce_bf16y(y16.reshape(40, 512), w)
+    assert st == 0 and st16 == 0 and np.array_equal(got, want)
+    assert not np.array_equal(got, O.reduce(y, w)[2])                             # and it is a different numerical mode
 
 
 # ---- activation ------------------------------------------------------------------------------------

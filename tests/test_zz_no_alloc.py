@@ -47,6 +47,24 @@ def test_static_workspace_call_equals_the_allocating_call():
         assert status[0] == stats.groups and status[2] > 0 and not status[[1, 3, 4, 6, 7]].any() and status[5] == 0xFFFFFFFF, status
 
 
+def test_static_workspace_call_allocates_nothing():
+    """The GPU's free memory reads the same before and after calls of the entry, the first call on this GPU
+    included when this test runs alone (the workspace is part of the loaded code object, not an allocation),
+    and the array needs no initialising call: its constants are rewritten by every call's first kernel."""
+    wl = synth.make(2)
+    layer = DeviceLayer(wl.pools(wl.touched())).layer
+    bufs = device_inputs(wl)
+    out, status = b1.DeviceBuffer(wl.rows * 4096 * 2), b1.DeviceBuffer(32)
+    out.to_host(np.uint16)                                           # the library is loaded and the device initialised by now
+    free_before = b1.device_memory()[0]
+    for rows in (wl.rows, 16):
+        b1.ffn_static(layer, bufs[0].ptr, 4096, bufs[1].ptr, 128, bufs[2].ptr, bufs[3].ptr, rows, out.ptr, status.ptr)
+        assert b1.device_memory()[0] == free_before
+    words = status.to_host(np.uint32)
+    assert words[0] > 0 and not words[[1, 3, 4, 6, 7]].any()
+    assert b1.device_memory()[0] == free_before
+
+
 def test_static_workspace_limits_and_status_words():
     wl = synth.make(2)
     layer = DeviceLayer(wl.pools(wl.touched())).layer
