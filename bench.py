@@ -30,6 +30,10 @@ NOMINAL_GHZ = 2.4               # the engine clock the published peaks are quote
 # one the profile holds, or null when the profile is not there.
 TRAFFIC_PROFILE = os.path.join("profiles", "hbm_traffic_decode128_prefill8192.md")
 PREFILL_WARMUP, PREFILL_SAMPLES = 10, 31   # the reference's timing protocol (tests/b1_core/bench_connected.cuh:73-81)
+PARITY_TOKENS = 64                          # rows checked against the CPU rule on both sides of every timed region
+RANK_LAYER_BYTES = 855_638_016              # 256 quarter-slice images: the gate's unique weight and scale bytes
+# The reference's gate (crates/mimo26-expert/src/bench.rs:41-48): at least 70 % of the memory peak at M <= 8, STOP below 60 %.
+GATE_TARGET, GATE_STOP = 0.70, 0.60
 
 
 def log(*a):
@@ -131,15 +135,25 @@ def kernel_phases(layer, scratch, d, rows, reps, b1):
                 fc1=spread(a[:, 1]), fc2=spread(a[:, 2]), reduce=spread(a[:, 3]), plan=spread(a[:, 0]))
 
 
-def sample_parity(wl, pools, got_bits, tokens, O):
-    """GPU BF16 rows against the CPU checker's BF16 rows on a few tokens (like with like: both sides
-    carry the one BF16 rounding of the rank sum)."""
-    ref_rc, _, ref_bits, _ = O.layer_ffn(pools, wl.payload[tokens], wl.scales[tokens], wl.ids[tokens], wl.weights[tokens])
-    got = (got_bits[tokens].astype(np.uint32) << 16).view(np.float32).astype(np.float64)
+def bars(got_bits, ref_bits):
+    """max-abs / max|ref| and mean relative error of BF16 rows against the CPU checker's BF16 rows."""
+    got = (got_bits.astype(np.uint32) << 16).view(np.float32).astype(np.float64)
     ref = (ref_bits.astype(np.uint32) << 16).view(np.float32).astype(np.float64)
-    return dict(tokens=len(tokens), oracle_rc=ref_rc, max_abs_over_max_ref=float(np.max(np.abs(got - ref)) / np.max(np.abs(ref))),
+    return dict(max_abs_over_max_ref=float(np.max(np.abs(got - ref)) / np.max(np.abs(ref))),
                 mean_rel=float(np.sum(np.abs(got - ref)) / np.sum(np.abs(ref))),
-                bf16_identical_fraction=float(np.mean(got_bits[tokens] == ref_bits)))
+                bf16_identical_fraction=float(np.mean(got_bits == ref_bits)))
+
+
+def sample_parity(wl, pools, before_bits, after_bits, tokens, O):
+    """GPU BF16 rows against the CPU checker's BF16 rows on `tokens` (like with like: both sides carry the one
+    BF16 rounding of the rank sum), for the output taken before the timed region and the one taken after it
+    (the reference's gate validates on both sides of its timing, tests/b1_core/bench_connected.cuh:56-63,85)."""
+    ref_rc, _, ref_bits, _ = O.layer_ffn(pools, wl.payload[tokens], wl.scales[tokens], wl.ids[tokens], wl.weights[tokens])
+    out = dict(tokens=len(tokens), oracle_rc=ref_rc, **bars(after_bits[tokens], ref_bits))
+    out["before_timing"] = bars(before_bits[tokens], ref_bits)
+    out["within_bars_before_and_after"] = bool(ref_rc == 0 and all(b["max_abs_over_max_ref"] <= 1e-2 and b["mean_rel"] <= 1e-3
+                                                                   for b in (out, out["before_timing"])))
+    return out
 
 
 def cpu_baseline(wl, pools, tokens, O):
@@ -167,9 +181,10 @@ def cpu_baseline(wl, pools, tokens, O):
     return out
 
 
-def run_config(cfg, steps, warmup, torch, dev, b1, synth, O, parity_tokens, cpu_tokens, samples=0):
+def run_config(cfg, steps, warmup, torch, dev, b1, synth, O, parity_tokens, cpu_tokens, samples=0, variants=()):
     """Correctness before and after the timing, as the reference's bench gate does. `samples` > 0 adds the
-    per-step event protocol (that many single steps after `warmup` warm-ups: median / min / max)."""
+    per-step event protocol (that many single steps after `warmup` warm-ups: median / min / max). `variants`:
+    scratch options whose step is sampled beside the default (never the headline)."""
     wl = synth.make(cfg)
     log(f"[bench] config {cfg}: {wl.name}")
     layer, pools = build_layer(wl, torch, dev, b1)
@@ -183,14 +198,98 @@ def run_config(cfg, steps, warmup, torch, dev, b1, synth, O, parity_tokens, cpu_
     ticks = scratch.view("clock", np.uint64, 4)  # the tile launches of the last call: shader-clock and 100 MHz ticks, FC1 then FC2
     ph["clock_ghz"] = [float(ticks[i]) / float(ticks[i + 1]) * 0.1 if ticks[i + 1] else None for i in (0, 2)]
     after = d["out"].cpu().numpy().view(np.uint16)
-    tokens = np.arange(min(parity_tokens, wl.rows))
-    par = sample_parity(wl, pools, after, tokens, O)
+    tokens = np.linspace(0, wl.rows - 1, min(parity_tokens, wl.rows)).astype(np.int64)  # spread over the batch
+    par = sample_parity(wl, pools, before, after, tokens, O)
     par["bitwise_stable_across_timing"] = bool(np.array_equal(before, after))
     cpu = cpu_baseline(wl, pools, np.arange(min(cpu_tokens, wl.rows)), O) if cpu_tokens else None
     touched = int(wl.touched().size)
     res = dict(wl=wl, ms_per_step=wall_ms, event_ms_per_step=ev_ms, per_step=per_step, phases=ph, parity=par, cpu=cpu, touched=touched)
+    res["variants"] = {}
+    for name in variants:  # same layer, same inputs, a scratch of its own with the option on
+        alt = b1.Scratch(stream=torch.cuda.current_stream().cuda_stream)
+        alt.set_option(name, True)
+        steps_ms = spread(sampled_steps(layer, alt, d, wl.rows, max(samples, PREFILL_SAMPLES), warmup, torch, b1))
+        alt_ph = kernel_phases(layer, alt, d, wl.rows, 11, b1)
+        got = d["out"].cpu().numpy().view(np.uint16)
+        ref_rc, _, ref_bits, _ = O.layer_ffn(pools, wl.payload[tokens], wl.scales[tokens], wl.ids[tokens], wl.weights[tokens])
+        res["variants"][name] = dict(ms_per_step=steps_ms["median"], ms_per_step_spread=steps_ms, fc2_ms=alt_ph["fc2"]["median"],
+                                     reduce_ms=alt_ph["reduce"]["median"], same_bits_as_default=bool(np.array_equal(got, after)),
+                                     parity_against_the_default_cpu_rule=dict(tokens=len(tokens), oracle_rc=ref_rc, **bars(got[tokens], ref_bits)))
+        alt.close()
     del layer, scratch
     return res
+
+
+def gate_workload(m, synth):
+    """The routing of the reference's bandwidth gate (tests/b1_core/bench_connected.cuh:7-12,47-50): 32 * m tokens,
+    every run of m tokens shares eight experts, the 32 runs cover all 256 experts exactly once, so every expert gets
+    m rows; weights (slot + 1) / 36. Activations: seeded N(0,1) rows through the wire quantizer (the reference
+    replays eight captured rows, which this image does not hold)."""
+    rows = 32 * m
+    perm = np.argsort(synth.uniform(synth.stream_key(synth.BASE_SEED + 60, synth.ROUTES), 256), kind="stable").astype(np.int32)
+    ids = perm.reshape(32, 8)[np.arange(rows) // m]
+    w = np.tile(np.arange(1, 9, dtype=np.float32) / 36, (rows, 1))
+    x = synth._activations(synth.BASE_SEED + 60, rows)
+    payload, scales = synth.q0_quantize(x)
+    return synth.Workload(f"gate M={m}", 1, synth.BASE_SEED + 1, 1, rows, ids, w, x, payload, scales)
+
+
+def run_rank_share(torch, dev, b1, synth, O):
+    """One TP4 rank's share (I = 512, the reference's deployment shape): configs[0] and configs[1] timed, and the
+    reference's own gate: 256 experts of one rank, M = 1..8 rows per expert, 10 warm-ups, 31 event samples,
+    median; the gate's timed scope is FC1 + SwiGLU + quantizer + FC2 (plan and combine outside it, reported
+    beside), its metric the rank layer's 855,638,016 unique weight and scale bytes over that time."""
+    out = {"shape": "256 experts x one TP4 rank's share (I 512), H 4096, top-8", "peak_GBps": HBM_PEAK_GBS}
+    wl1 = synth.make(1)
+    layer, pools = build_layer(synth.Workload("rank layer", 1, wl1.seed, 1, 0, wl1.ids, wl1.weights, wl1.x, wl1.payload, wl1.scales), torch, dev, b1)
+    scratch = b1.Scratch(stream=torch.cuda.current_stream().cuda_stream)
+
+    def timed(wl, parity_rows):
+        d = stage(wl, torch, dev)
+        kernel_phases(layer, scratch, d, wl.rows, 2, b1)
+        before = d["out"].cpu().numpy().view(np.uint16).copy()
+        steps = spread(sampled_steps(layer, scratch, d, wl.rows, PREFILL_SAMPLES, PREFILL_WARMUP, torch, b1))
+        ph = kernel_phases(layer, scratch, d, wl.rows, PREFILL_SAMPLES, b1)
+        after = d["out"].cpu().numpy().view(np.uint16)
+        tokens = np.linspace(0, wl.rows - 1, min(parity_rows, wl.rows)).astype(np.int64)
+        par = sample_parity(wl, pools, before, after, tokens, O)
+        par["bitwise_stable_across_timing"] = bool(np.array_equal(before, after))
+        return steps, ph, par
+
+    for cfg in (0, 1):
+        wl = synth.make(cfg)
+        steps, ph, par = timed(wl, wl.rows)  # every row
+        nbytes = wl.algorithmic_bytes()
+        gbs = nbytes / (steps["median"] * 1e-3) / 1e9
+        out[f"configs[{cfg}]"] = {"workload": wl.name, "experts_touched": int(wl.touched().size), "algorithmic_bytes": nbytes,
+                                  "ms_per_step": steps["median"], "ms_per_step_spread": steps, "GBps": gbs, "frac_of_hbm_peak": gbs / HBM_PEAK_GBS,
+                                  "tok_per_s": wl.rows / (steps["median"] * 1e-3), "flops": wl.flops(),
+                                  "plan_ms": ph["plan"]["median"], "fc1_ms": ph["fc1"]["median"], "fc2_ms": ph["fc2"]["median"],
+                                  "reduce_ms": ph["reduce"]["median"], "parity": par}
+    gate = []
+    scratch.set_option("scope_timing", True)  # FC1 + SwiGLU + quantizer + FC2 between two events, none between the stages
+    for m in range(1, 9):
+        wl = gate_workload(m, synth)
+        steps, ph, par = timed(wl, wl.rows if m in (1, 8) else 32)  # every row at both ends of the sweep, 32 rows between
+        scope_ms = ph["fc1"]["median"]
+        gbs = RANK_LAYER_BYTES / (scope_ms * 1e-3) / 1e9
+        frac = gbs / HBM_PEAK_GBS
+        gate.append({"M": m, "rows": wl.rows, "timed_scope_ms": scope_ms, "timed_scope_ms_spread": ph["fc1"],
+                     "plan_ms": ph["plan"]["median"], "reduce_ms": ph["reduce"]["median"], "whole_step_ms": steps["median"],
+                     "effective_unique_weight_GBps": gbs, "frac_of_hbm_peak": frac,
+                     "whole_step_GBps": (RANK_LAYER_BYTES + wl.rows * (4224 + 64 + 8192)) / (steps["median"] * 1e-3) / 1e9,
+                     "verdict": "TARGET" if frac >= GATE_TARGET else "STOP" if frac < GATE_STOP else "PIVOT", "parity": par})
+    out["gate"] = {"protocol": "reference gate, crates/mimo26-expert/tests/b1_core/bench_connected.cuh:21-88: all 256 experts of one rank, M rows "
+                               "per expert, 10 warm-ups, 31 event samples, median; timed scope FC1 + SwiGLU + quantizer + FC2 (per-kernel events of "
+                               "the library, each carrying about 3 us of event), plan and combine beside it; metric 855,638,016 B / scope time; "
+                               "thresholds of crates/mimo26-expert/src/bench.rs:41-48 against 8 TB/s",
+                   "unique_weight_scale_bytes": RANK_LAYER_BYTES, "target_frac": GATE_TARGET, "stop_frac": GATE_STOP, "rows": gate,
+                   "reference_published_GB10_GBps": {"first_connected_run_M1..8": [160.65, 160.05, 158.56, 157.13, 155.23, 153.68, 152.50, 152.78],
+                                                     "after_tuning_M<=8": 184.0, "GB10_peak": 273.0}}
+    scratch.close()
+    del layer
+    torch.cuda.empty_cache()
+    return out
 
 
 def stack_reference_rows(seed, layer, payload, scales, ids, weights, O, synth):
@@ -302,6 +401,11 @@ def main():
     ap.add_argument("--only-prefill", action="store_true",
                     help="profiling aid: run only the prefill measurement and print its object")
     ap.add_argument("--no-stack", action="store_true", help="skip the 48-layer resident stack (configs[4]) object")
+    ap.add_argument("--no-rank-share", action="store_true", help="skip the rank-share object (configs[0], configs[1], the reference's gate sweep)")
+    ap.add_argument("--only-rank-share", action="store_true", help="profiling aid: run only the rank-share leg and print its object")
+    ap.add_argument("--no-variants", action="store_true",
+                    help="profiling aid: skip the opt-in forms (fused combine, BF16 per-route rows) sampled beside the default, so a kernel "
+                         "trace of the run holds the default path's launches only")
     ap.add_argument("--stack", type=int, default=0, metavar="LAYERS",
                     help="run configs[4] instead: this many layers' routed experts resident in HBM (48 = the full model, 164 GB)")
     ap.add_argument("--stack-tokens", type=int, default=65536, help="prefill length of the --stack run (a multiple of 4096)")
@@ -328,12 +432,15 @@ def main():
         torch.cuda.synchronize()
         del src, dst
         torch.cuda.empty_cache()
+    if args.only_rank_share:
+        print(json.dumps(run_rank_share(torch, dev, b1, synth, O)), flush=True)
+        return
     if args.only_prefill:
-        pre = run_config(3, args.steps, args.warmup, torch, dev, b1, synth, O, parity_tokens=2, cpu_tokens=0)
+        pre = run_config(3, args.steps, args.warmup, torch, dev, b1, synth, O, parity_tokens=PARITY_TOKENS, cpu_tokens=0)
         print(json.dumps(dict(ms_per_step=pre["ms_per_step"], phases=pre["phases"], parity=pre["parity"])), flush=True)
         return
-    dec = run_config(2, args.steps, args.warmup, torch, dev, b1, synth, O, parity_tokens=8,
-                     cpu_tokens=0 if args.no_cpu else 128, samples=PREFILL_SAMPLES)
+    dec = run_config(2, args.steps, args.warmup, torch, dev, b1, synth, O, parity_tokens=PARITY_TOKENS,
+                     cpu_tokens=0 if args.no_cpu else 128, samples=PREFILL_SAMPLES, variants=() if args.no_variants else ("fused_combine",))
     wl = dec["wl"]
     inter, U = wl.intermediate, dec["touched"]
     # Algorithmic bytes: unique weight bytes of the touched experts + input rows + ids/weights + BF16 rows;
@@ -363,6 +470,7 @@ def main():
                               "fc2_ms_spread": dec["phases"]["fc2"], "per_step_ms": dec["per_step"]}},
         "cpu_baseline": dec["cpu"],
         "parity": dec["parity"],
+        "fused_combine": dec["variants"].get("fused_combine"),   # opt-in form of the combine: same bits, beside the default
     }
     # The same figures against what this box sustains: a streaming read of 4 GiB, and the GEMMs' MFMA alone.
     from mimo26f_afd_amd import probe
@@ -374,7 +482,8 @@ def main():
     if not args.no_prefill:
         # The reference's protocol: at least 10 warm-ups, at least 31 single-step event samples, the median reported.
         p_warm, p_samples = max(PREFILL_WARMUP, args.warmup), max(PREFILL_SAMPLES, args.steps)
-        pre = run_config(3, p_samples, p_warm, torch, dev, b1, synth, O, parity_tokens=4, cpu_tokens=0, samples=p_samples)
+        pre = run_config(3, p_samples, p_warm, torch, dev, b1, synth, O, parity_tokens=PARITY_TOKENS, cpu_tokens=0, samples=p_samples,
+                         variants=() if args.no_variants else ("bf16_route_rows", "fused_combine"))
         pw = pre["wl"]
         flops = pw.flops()
         step_ms = pre["per_step"]["median"]
@@ -395,7 +504,14 @@ def main():
                                   "plan_ms": pre["phases"]["plan"]["median"], "fc2_ms": pre["phases"]["fc2"]["median"],
                                   "reduce_ms": pre["phases"]["reduce"]["median"], "fc2_ms_spread": pre["phases"]["fc2"]}},
             "parity": pre["parity"],
+            # Opt-in forms, never the headline: the reference's MIMO26_B1_Y=bf16 numerical mode (per-route rows kept
+            # as BF16: not the default mode's bits) and the combine inside FC2 (the default mode's bits).
+            "bf16_route_rows": pre["variants"].get("bf16_route_rows"),
+            "fused_combine": pre["variants"].get("fused_combine"),
         }
+        for v in ("bf16_route_rows", "fused_combine"):
+            if line["prefill"][v]:
+                line["prefill"][v]["path_frac_of_fp8_peak"] = flops / (line["prefill"][v]["ms_per_step"] * 1e-3) / 1e12 / MFMA_FP8_PEAK_TFLOPS
         mfma_tf = probe.mfma_rate_tflops()
         line["prefill"]["roofline"]["measured_mfma_TFLOPs"] = mfma_tf
         line["prefill"]["roofline"]["frac_of_measured"] = fc1_tf / mfma_tf
@@ -412,6 +528,13 @@ def main():
             "mfma_only_TFLOPs_after_40_launches": held["tflops_last"]}
         if fc1_ghz:
             line["prefill"]["roofline"]["frac_at_clock"] = fc1_tf / (MFMA_FP8_PEAK_TFLOPS * fc1_ghz / NOMINAL_GHZ)
+    if not args.no_rank_share:
+        try:
+            t0 = time.time()
+            line["rank_share"] = run_rank_share(torch, dev, b1, synth, O)
+            line["rank_share"]["leg_seconds"] = time.time() - t0
+        except Exception as e:  # the headline line must survive a failure of this leg
+            line["rank_share"] = {"error": f"{type(e).__name__}: {e}"}
     if not args.no_stack:
         # configs[4] with all 48 layers resident needs about 175 GiB of HBM; without it the object says so.
         free_gib = torch.cuda.mem_get_info()[0] / 2**30

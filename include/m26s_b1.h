@@ -153,19 +153,27 @@ void m26s_b1_scratch_set_taps(m26s_b1_scratch* scratch, int on);
 /* Switches of a scratch, for the calls made on it afterwards. Returns 0, 1 for a bad handle or option, 2 for
  * a runtime error.
  *   TAPS              as m26s_b1_scratch_set_taps.
- *   SEPARATE_COMBINE  the router-weighted combine runs as a launch of its own behind FC2
- *                     (crates/mimo26-spark/kernels/b1_serve.cu:502-515 launches it so). By default FC2 does it:
- *                     the wave that writes a token's eighth per-route row sums the eight, in slot order, so
- *                     both forms give the same bits. Layers on the conforming arm always combine separately.
+ *   FUSED_COMBINE     the router-weighted combine runs inside FC2 instead of as a launch of its own behind it
+ *                     (crates/mimo26-spark/kernels/b1_serve.cu:502-515 launches it): the wave that writes a
+ *                     token's eighth per-route row sums the eight, in slot order, so both forms give the same
+ *                     bits (tested). Off by default: measured on MI355X it is never the faster form (level at
+ *                     16 tokens of one rank's share, 2 % behind at 128 tokens, 5 % at 8192: a wave's waits for
+ *                     its stores, its count and the rows it sums are paid with nothing else to run). Layers on
+ *                     the conforming arm always combine separately.
  *   BF16_ROUTE_ROWS   the reference's opt-in MIMO26_B1_Y=bf16 (b1_serve.cu:98-143,400-405; the store rule of
  *                     crates/mimo26-expert/kernels/b1/connected.cu:41-44): FC2 keeps its per-route rows as
  *                     BF16 bits instead of FP32 and the combine widens them. A numerical-mode change, never
  *                     the default; a scratch is created with it on when the environment holds MIMO26_B1_Y=bf16.
  *                     View 7 then holds uint16 rows.
+ *   SCOPE_TIMING      the timed entries record one interval over FC1 + SwiGLU + quantizer + FC2 with no event between
+ *                     the stages, the scope the reference's bandwidth gate times between its two events
+ *                     (crates/mimo26-expert/tests/b1_core/bench_connected.cuh:66-81): ms[4] is then that interval
+ *                     and ms[6] is 0. An event is one more packet between two dependent kernels, about 3 us.
  *   GUARDS            test aid (the counterpart of crates/mimo26-expert/tests/b1_core/primitive.cu:23-40):
  *                     every internal array is followed, and the first preceded, by at least 256 bytes of 0xa5,
  *                     written before each call and read back by m26s_b1_scratch_check_guards. */
-enum { M26S_B1_OPT_TAPS = 0, M26S_B1_OPT_SEPARATE_COMBINE = 1, M26S_B1_OPT_BF16_ROUTE_ROWS = 2, M26S_B1_OPT_GUARDS = 3 };
+enum { M26S_B1_OPT_TAPS = 0, M26S_B1_OPT_FUSED_COMBINE = 1, M26S_B1_OPT_BF16_ROUTE_ROWS = 2, M26S_B1_OPT_GUARDS = 3,
+       M26S_B1_OPT_SCOPE_TIMING = 4 };
 int m26s_b1_scratch_set_option(m26s_b1_scratch* scratch, int option, int value);
 /* Waits for the scratch's stream and reads every red zone back: 0 intact, 1 guards not enabled or no call made,
  * 2 runtime error, 4 a zone holds a byte other than 0xa5 (err names the zone and the offset). */

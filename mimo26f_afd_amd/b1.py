@@ -103,15 +103,16 @@ class Scratch:
         else:
             _raise(load().m26s_b1_scratch_new_on(stream, C.byref(self._h), buf, ERRLEN), buf)
 
-    OPTION = dict(taps=0, separate_combine=1, bf16_route_rows=2, guards=3)
+    OPTION = dict(taps=0, fused_combine=1, bf16_route_rows=2, guards=3, scope_timing=4)
 
     def set_taps(self, on: bool) -> None:
         load().m26s_b1_scratch_set_taps(self._h, 1 if on else 0)
 
     def set_option(self, name: str, on: bool) -> None:
-        """Switches for the calls that follow: 'separate_combine' (the combine as a launch of its own instead of
-        inside FC2; same bits), 'bf16_route_rows' (the reference's opt-in MIMO26_B1_Y=bf16 numerical mode),
-        'guards' (red zones around every internal array, read back by check_guards), 'taps'."""
+        """Switches for the calls that follow: 'fused_combine' (the combine inside FC2 instead of as a launch of its
+        own; same bits, not faster), 'bf16_route_rows' (the reference's opt-in MIMO26_B1_Y=bf16 numerical mode),
+        'guards' (red zones around every internal array, read back by check_guards), 'scope_timing' (the timed
+        entries report FC1 + FC2 as one interval in phase_ms[0]), 'taps'."""
         rc = load().m26s_b1_scratch_set_option(self._h, self.OPTION[name], 1 if on else 0)
         if rc:
             raise B1Error(rc, f"b1 scratch: option {name} refused")

@@ -226,7 +226,7 @@ struct m26s_b1_scratch {
     uint8_t* slab = nullptr;
     size_t slab_bytes = 0;
     Workspace last{};  // of the latest call, for the views
-    bool taps = false, separate_combine = false, y_bf16 = false, guards = false;
+    bool taps = false, fused_combine = false, y_bf16 = false, guards = false, scope_timing = false;
     uint32_t last_rows = 0;
     uint8_t* bounce = nullptr;  // page-locked host staging for callers whose own arrays are pageable
     size_t bounce_bytes = 0;
@@ -249,7 +249,7 @@ int fit_slab(m26s_b1_scratch* S, size_t bytes, bool& grew, Outcome& out) {
 
 Shape shape_of(const m26s_b1_layer* L, const m26s_b1_scratch* S, uint32_t rows, bool host_io) {
     const bool conforming = !L->all_normal;
-    return Shape{rows, L->lay.inter, S->taps, host_io, conforming, !S->separate_combine && !conforming, S->y_bf16, S->guards};
+    return Shape{rows, L->lay.inter, S->taps, host_io, conforming, S->fused_combine && !conforming, S->y_bf16, S->guards};
 }
 
 // Sizes the slab for the call and lays the call's arrays out in it (S->last).
@@ -421,7 +421,7 @@ int enqueue(const m26s_b1_layer* L, m26s_b1_scratch* S, bool host_io, bool timed
         M26G_TRY(out, hipGetLastError(), "b1 red zones");
     }
     const Launch k{S->stream, fixed_at(S->fixed), S->last, S->taps, S->y_bf16, timed ? S->planned : nullptr,
-                   timed ? S->fc1_done : nullptr, timed ? S->fc2_done : nullptr};
+                   timed && !S->scope_timing ? S->fc1_done : nullptr, timed ? S->fc2_done : nullptr};
     if (host_io) {  // the inputs were staged into the slab by the caller of this function
         x = S->last.x, xp = kHidden, xs = S->last.xs, xsp = kHidden / 32, ids = S->last.ids, w = S->last.weights;
         bf16_out = S->last.bf16;
@@ -472,8 +472,12 @@ void report(m26s_b1_scratch* S, float* ms, float host_front, float host_total, u
     float plan = 0, gpu = 0, fc1 = 0, fc2 = 0, combine = 0;
     (void)hipEventElapsedTime(&plan, S->begun, S->planned);
     (void)hipEventElapsedTime(&gpu, S->planned, S->ended);
-    (void)hipEventElapsedTime(&fc1, S->planned, S->fc1_done);
-    (void)hipEventElapsedTime(&fc2, S->fc1_done, S->fc2_done);
+    if (S->scope_timing) {  // one interval over both GEMM stages, no event between them
+        (void)hipEventElapsedTime(&fc1, S->planned, S->fc2_done);
+    } else {
+        (void)hipEventElapsedTime(&fc1, S->planned, S->fc1_done);
+        (void)hipEventElapsedTime(&fc2, S->fc1_done, S->fc2_done);
+    }
     (void)hipEventElapsedTime(&combine, S->fc2_done, S->ended);
     const float tail = host_total - host_front - plan - gpu;
     const float v[8] = {host_front + plan, gpu, tail < 0 ? 0 : tail, float(groups), fc1, 0.0f, fc2, combine};
@@ -742,7 +746,7 @@ int m26s_b1_ffn_static(const m26s_b1_layer* L, const uint8_t* payload_dev, size_
         return out.fail(1, "b1 ffn: bad rows/handles/pitch");
     if (rows > kStaticRows)
         return out.fail(1, "b1 ffn static: %u rows exceed the %u rows the fixed workspace holds", rows, kStaticRows);
-    const Shape shape{rows, L->lay.inter, false, false, !L->all_normal, L->all_normal, false, false};
+    const Shape shape{rows, L->lay.inter, false, false, !L->all_normal, false, false, false};
     if (carve(nullptr, shape).total + kFixedBytes > kStaticBytes)
         return out.fail(1, "b1 ffn static: the call needs more than the fixed workspace of %zu bytes", kStaticBytes);
     const hipStream_t stream = static_cast<hipStream_t>(hip_stream);
@@ -775,8 +779,9 @@ int m26s_b1_scratch_set_option(m26s_b1_scratch* S, int option, int value) {
     const bool on = value != 0;
     switch (option) {
     case M26S_B1_OPT_TAPS: S->taps = on; return 0;
-    case M26S_B1_OPT_SEPARATE_COMBINE: S->separate_combine = on; return 0;
+    case M26S_B1_OPT_FUSED_COMBINE: S->fused_combine = on; return 0;
     case M26S_B1_OPT_BF16_ROUTE_ROWS: S->y_bf16 = on; return 0;
+    case M26S_B1_OPT_SCOPE_TIMING: S->scope_timing = on; return 0;
     case M26S_B1_OPT_GUARDS:
         if (S->guards != on) {  // the layout changes: the next call starts on a fresh slab, armed again
             if (hipStreamSynchronize(S->stream) != hipSuccess) return 2;

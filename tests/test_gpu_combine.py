@@ -1,9 +1,9 @@
 """The router-weighted combine on the GPU in its three forms, through the C ABI.
 
-Default: fused into FC2 (the wave that writes a token's eighth per-route row sums the eight, in slot order).
-`separate_combine`: a launch of its own behind FC2, as the reference runs it
-(crates/mimo26-spark/kernels/b1_serve.cu:502-515). The two must give the same bits everywhere: the sum's order
-is fixed by the slots, and integer counts decide only which wave performs it.
+Default: a launch of its own behind FC2, as the reference runs it
+(crates/mimo26-spark/kernels/b1_serve.cu:502-515). `fused_combine`: inside FC2 (the wave that writes a token's
+eighth per-route row sums the eight, in slot order). The two must give the same bits everywhere: the sum's
+order is fixed by the slots, and integer counts decide only which wave performs it.
 `bf16_route_rows`: the reference's opt-in numerical mode MIMO26_B1_Y=bf16 (b1_serve.cu:98-143,400-405),
 against the CPU rule for it (orc_bf16_store_rows, orc_reduce_bf16y), bit for bit on the GPU's own rows.
 """
@@ -24,10 +24,10 @@ def subset(wl, pick, name):
 
 def both_forms(layer, wl):
     fused, apart = b1.Scratch(), b1.Scratch()
-    apart.set_option("separate_combine", True)
+    fused.set_option("fused_combine", True)
     s1, bf1, pf1 = run_ffn_dev(layer, fused, wl)
     s2, bf2, pf2 = run_ffn_dev(layer, apart, wl)
-    if wl.rows >= 4096:  # no combine launch in the default form: nothing lies between the FC2 event and the end event
+    if wl.rows >= 4096:  # no combine launch in the fused form: nothing lies between the FC2 event and the end event
         assert s1.phase_ms[3] < 0.02 < s2.phase_ms[3], (s1.phase_ms, s2.phase_ms)
     y1 = fused.view("y", np.float32, wl.rows * 8 * 4096)
     y2 = apart.view("y", np.float32, wl.rows * 8 * 4096)
@@ -72,14 +72,14 @@ def test_fused_combine_on_the_whole_prefill_chunk(full_layer):
 
 
 def test_fused_combine_reports_the_combine_fault(full_layer):
-    """A sum that leaves binary32's finite range raises the combine's fault word from inside FC2, as the separate
-    launch does (return code 4, 'reduce fault')."""
+    """A sum that leaves binary32's finite range raises the combine's fault word, from the separate launch and
+    from inside FC2 alike (return code 4, 'reduce fault')."""
     wl, _, layer = full_layer
     few = subset(wl, np.arange(4), "overflowing weights")
     few.weights[:] = np.float32(3.0e38)                                  # legal weights (finite, non-negative) whose products overflow
-    for separate in (False, True):
+    for fuse in (False, True):
         s = b1.Scratch()
-        s.set_option("separate_combine", separate)
+        s.set_option("fused_combine", fuse)
         with pytest.raises(b1.B1Error, match="reduce fault") as e:
             run_ffn_dev(layer, s, few)
         assert e.value.code == 4
@@ -98,14 +98,14 @@ def test_bf16_route_rows_mode(full_layer):
         want_rows = O.bf16_store_rows(y32)
         st, want = O.reduce_bf16y(want_rows, case.weights)
         assert st == 0
-        for separate in (False, True):
+        for fuse in (False, True):
             s = b1.Scratch()
             s.set_option("bf16_route_rows", True)
-            s.set_option("separate_combine", separate)
+            s.set_option("fused_combine", fuse)
             _, bf, _ = run_ffn_dev(layer, s, case, want_partial=False)
             rows16 = s.view("y", np.uint16, case.rows * 8 * 4096).reshape(case.rows * 8, 4096)
-            assert np.array_equal(rows16, want_rows), (case.name, separate)
-            assert np.array_equal(bf, want), (case.name, separate)
+            assert np.array_equal(rows16, want_rows), (case.name, fuse)
+            assert np.array_equal(bf, want), (case.name, fuse)
         assert not np.array_equal(bf, bf_plain)                              # a numerical-mode change, not the default
         rc, _, ref_bf16, _ = O.layer_ffn(pools, case.payload, case.scales, case.ids, case.weights)
         ma, mr = parity(bf16_to_f32(bf), bf16_to_f32(ref_bf16))
