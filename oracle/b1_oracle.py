@@ -36,7 +36,8 @@ class _Layer(C.Structure):
 
 def _load():
     build()
-    lib = C.CDLL(os.path.join(HERE, "liboracle.so"))
+    # B1_ORACLE_LIB: another build of the same checker (the sanitized one of `make -C oracle asan`)
+    lib = C.CDLL(os.environ.get("B1_ORACLE_LIB") or os.path.join(HERE, "liboracle.so"))
     lib.orc_mxfp4_bits.restype = C.c_uint32
     lib.orc_mxfp4_bits.argtypes = [C.c_uint32, C.c_uint32]
     lib.orc_e4m3_value.restype = C.c_float
