@@ -18,6 +18,12 @@ and this module checks them on the assembly hipcc emits (no GPU needed):
     hand-written MFMA and the next non-MFMA access to its destination, and wants at least 16
     (the compiler's own hazard tables hold 8 passes + 3 for this MFMA; the rest is margin).
 
+ 4. in every kernel of the library, a store of more than eight bytes written as an `asm` statement is
+    followed, inside the same statement, by at least two wait states (`s_nop 1`). Such a store reads the
+    upper half of its data a little after it issues; the compiler keeps the next instructions off those
+    registers for the stores it emits itself, and cannot for one it does not recognise (it reused the
+    registers at once, and two of four stored columns came out wrong now and then).
+
 "In flight" follows the hardware's counters. Vector-memory operations (loads, stores, direct-to-LDS
 loads, whoever issued them) complete in issue order, and `s_waitcnt vmcnt(N)` returns when at most N
 are outstanding: an operation has landed behind such a wait exactly when at least N younger ones were
@@ -250,6 +256,27 @@ def check(asm_text: str) -> tuple[dict, list]:
     return seen, problems
 
 
+WIDE_STORE = re.compile(r"^(global|buffer|flat|scratch)_store_dwordx[34]\b")
+
+
+def check_asm_stores(asm_text: str) -> tuple[int, list]:
+    """Rule 4 over the whole file: (wide stores found inside asm statements, problems)."""
+    found, problems, inasm, lines = 0, [], False, asm_text.splitlines()
+    for n, line in enumerate(lines):
+        text = line.strip()
+        if "ASMSTART" in text:
+            inasm = True
+        elif "ASMEND" in text:
+            inasm = False
+        elif inasm and WIDE_STORE.match(text):
+            found += 1
+            nxt = lines[n + 1].strip() if n + 1 < len(lines) else ""
+            m = re.match(r"s_nop\s+(\d+)", nxt)
+            if not m or int(m.group(1)) < 1:
+                problems.append(f"line {n + 1}: asm store of more than eight bytes without its wait states: {text}")
+    return found, problems
+
+
 def compile_to_asm() -> str:
     with tempfile.TemporaryDirectory() as tmp:
         out = os.path.join(tmp, "b1_abi.s")
@@ -264,9 +291,15 @@ def compile_to_asm() -> str:
 
 def run() -> dict:
     """Compile, check, raise on any problem; returns the per-kernel count of hand-issued loads."""
-    seen, problems = check(compile_to_asm())
+    text = compile_to_asm()
+    seen, problems = check(text)
     if len(seen) < 3 or min(seen.values()) < 100:
         raise RuntimeError(f"codegen check: tile kernels not found in the assembly ({seen})")
+    stores, store_problems = check_asm_stores(text)
+    if not stores:
+        raise RuntimeError("codegen check: the asm stores of the per-route rows were not found in the assembly")
+    problems += store_problems
+    seen["asm stores of more than eight bytes"] = stores
     if problems:
         raise RuntimeError("codegen check failed:\n" + "\n".join(problems[:12]))
     return seen

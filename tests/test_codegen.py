@@ -103,6 +103,23 @@ def test_checker_follows_the_control_flow():
     assert p == []
 
 
+def test_checker_wants_wait_states_inside_an_asm_store_of_more_than_eight_bytes():
+    """A store of more than eight bytes reads the upper half of its data after it issues; written as an asm
+    statement it has to bring its own two wait states, inside the statement."""
+    bare = ";;#ASMSTART\n\tglobal_store_dwordx4 v[0:1], v[14:17], off sc1\n\t;;#ASMEND\n\tv_mov_b32_e32 v16, 0"
+    n, p = codegen_check.check_asm_stores(bare)
+    assert n == 1 and len(p) == 1 and "wait states" in p[0]
+    for nop, problems in (("s_nop 1", 0), ("s_nop 0", 1), ("s_nop 3", 0)):
+        good = f";;#ASMSTART\n\tglobal_store_dwordx4 v[0:1], v[14:17], off sc1\n\t{nop}\n\t;;#ASMEND"
+        n, p = codegen_check.check_asm_stores(good)
+        assert n == 1 and len(p) == problems
+    # stores the compiler emitted itself (outside asm statements) and narrow asm stores are not its business
+    n, p = codegen_check.check_asm_stores("\tglobal_store_dwordx4 v[0:1], v[14:17], off\n;;#ASMSTART\n\tglobal_store_dwordx2 v[0:1], v[2:3], off sc1\n;;#ASMEND")
+    assert n == 0 and p == []
+
+
 def test_built_tile_kernels_pass():
     seen = codegen_check.run()
+    stores = seen.pop("asm stores of more than eight bytes")
+    assert stores >= 4                                                    # the per-route rows' stores of every FC2 body
     assert len(seen) == 3 and all(n >= 100 for n in seen.values())
