@@ -120,8 +120,10 @@ int m26s_b1_scratch_sync(m26s_b1_scratch* scratch, char* err, size_t errlen);
  * fault, lowest faulting block, fc2 fault, reduce fault} behind its last kernel: read them after the
  * stream has run; bf16_out_dev is valid when words 1, 3, 4, 6 and 7 are zero (decoded as m26s_b1_ffn's
  * return codes 3 and 4). All calls on one GPU share the one array, which keeps the last call's contents
- * (each call clears the words it needs at zero itself): calls that overlap in time on one GPU race, also
- * from different streams or threads. Pointers, pitches and alignments as m26s_b1_ffn_enqueue. */
+ * (each call's first kernel clears the words it needs at zero and rewrites the constants the array holds,
+ * so there is no initialising call that a graph capture could swallow: the first call on a GPU may be
+ * captured, and may come on any stream): calls that overlap in time on one GPU race, also from different
+ * streams or threads. Pointers, pitches and alignments as m26s_b1_ffn_enqueue. */
 int m26s_b1_ffn_static(const m26s_b1_layer* layer, const uint8_t* payload_dev, size_t payload_pitch,
                        const uint8_t* scales_dev, size_t scales_pitch, const int32_t* ids_dev,
                        const float* weights_dev, uint32_t rows, uint16_t* bf16_out_dev, uint32_t* status_dev,
