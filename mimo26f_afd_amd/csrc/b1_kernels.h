@@ -150,21 +150,32 @@ plan_kernel(const int32_t* __restrict__ ids, const float* __restrict__ w, uint32
     __shared__ uint8_t present[256];
     const uint32_t tid = threadIdx.x, lane = tid & 63, wv = tid >> 6, routes = rows * kTopk;
 
+    // Validation keys order faults as the serial planner meets them: (route + 1) << 4 | check,
+    // check 1 = id or residency, 2 = weight, 3 = expert repeated inside the token.
+    // One token (its eight routes) per thread and trip, two trips in flight: the walk is bound by the
+    // latency of these loads, not by their volume. The first trip's loads are asked for ahead of everything else
+    // (the checks need the residency bytes in LDS first): one memory latency for both instead of one after the other.
+    typedef v4i __attribute__((aligned(4))) v4i_u;
+    typedef v4f __attribute__((aligned(4))) v4f_u;
+    const v4i_u* ids4 = reinterpret_cast<const v4i_u*>(ids);
+    const v4f_u* w4 = reinterpret_cast<const v4f_u*>(w);
+    struct Trip { v4i ia, ib, ic, id; v4f wa, wb, wc, wd; };
+    auto fetch = [&](uint32_t t) {
+        const uint32_t u = t + kPlanThreads;
+        const bool two = u < rows;
+        return Trip{ids4[2 * t], ids4[2 * t + 1], ids4[two ? 2 * u : 2 * t], ids4[two ? 2 * u + 1 : 2 * t + 1],
+                    w4[2 * t], w4[2 * t + 1], w4[two ? 2 * u : 2 * t], w4[two ? 2 * u + 1 : 2 * t + 1]};
+    };
+    Trip first{};
+    if (tid < rows) first = fetch(tid);
+    const uint8_t here = tid < 256 ? resident[tid] : uint8_t(0);
     for (uint32_t i = tid; i < kPlanWaves * 256; i += kPlanThreads) (&hist[0][0])[i] = 0;
     if (tid == 0) first_bad = 0xffffffffu;
+    if (tid < 256) present[tid] = here;
     if (p.done)  // every call starts its completion counts from zero, whatever the call before left
         for (uint32_t i = tid; i < rows * kDoneBlocks; i += kPlanThreads) p.done[i] = 0;
     __syncthreads();
-    // Validation keys order faults as the serial planner meets them: (route + 1) << 4 | check,
-    // check 1 = id or residency, 2 = weight, 3 = expert repeated inside the token.
-    if (tid < 256) {
-        const uint8_t here = resident[tid];
-        if (here > 1) atomicMin(&first_bad, 1u);
-        present[tid] = here;
-    }
-    __syncthreads();
-    // One token (its eight routes) per thread and trip, two trips in flight: the walk is bound by the
-    // latency of these loads, not by their volume.
+    if (here > 1) atomicMin(&first_bad, 1u);
     auto check_token = [&](uint32_t t, const v4i& ia, const v4i& ib, const v4f& wa, const v4f& wb) {
         const int32_t e8[8] = {ia.x, ia.y, ia.z, ia.w, ib.x, ib.y, ib.z, ib.w};
         const float w8[8] = {wa.x, wa.y, wa.z, wa.w, wb.x, wb.y, wb.z, wb.w};
@@ -180,19 +191,10 @@ plan_kernel(const int32_t* __restrict__ ids, const float* __restrict__ w, uint32
         }
         *reinterpret_cast<uint2*>(id_byte + t * 8) = uint2{packed[0], packed[1]};
     };
-    typedef v4i __attribute__((aligned(4))) v4i_u;
-    typedef v4f __attribute__((aligned(4))) v4f_u;
-    const v4i_u* ids4 = reinterpret_cast<const v4i_u*>(ids);
-    const v4f_u* w4 = reinterpret_cast<const v4f_u*>(w);
     for (uint32_t t = tid; t < rows; t += 2 * kPlanThreads) {
-        const uint32_t u = t + kPlanThreads;
-        const bool two = u < rows;
-        const v4i ia = ids4[2 * t], ib = ids4[2 * t + 1];
-        const v4f wa = w4[2 * t], wb = w4[2 * t + 1];
-        const v4i ic = ids4[two ? 2 * u : 2 * t], id = ids4[two ? 2 * u + 1 : 2 * t + 1];
-        const v4f wc = w4[two ? 2 * u : 2 * t], wd = w4[two ? 2 * u + 1 : 2 * t + 1];
-        check_token(t, ia, ib, wa, wb);
-        if (two) check_token(u, ic, id, wc, wd);
+        const Trip trip = t == tid ? first : fetch(t);
+        check_token(t, trip.ia, trip.ib, trip.wa, trip.wb);
+        if (t + kPlanThreads < rows) check_token(t + kPlanThreads, trip.ic, trip.id, trip.wc, trip.wd);
     }
     __syncthreads();
     const uint32_t run = (((routes + kPlanWaves - 1) / kPlanWaves) + 63u) & ~63u;
