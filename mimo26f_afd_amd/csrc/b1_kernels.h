@@ -322,13 +322,18 @@ plan_kernel(const int32_t* __restrict__ ids, const float* __restrict__ w, uint32
 //                      expert, scans experts into route / group / chunk bases, fills group headers
 //                      and chunks, publishes the counts or the fault;
 //   plan_place_kernel  walks the routes again and places them.
+// The sum over earlier waves is taken in two levels: the count kernel, which holds its sixteen waves' counts in
+// LDS anyway, leaves every wave's start inside its own workgroup and the workgroup's totals; the scan turns the
+// totals (one row per workgroup, sixteen at 8192 rows) into every workgroup's start; the placement adds the two.
+// (Summed in one level by the scan alone, 256 rows of counts walked twice by one workgroup, the scan took 18 us.)
 // work: [0] first fault key (0xffffffff = none; the scan re-arms it), [1..3] unused,
-//       [4 ..) counts[wave][256], then route and group bases [2][257].
+//       [4 ..) starts[wave][256] inside the wave's workgroup, then totals[workgroup][256] (which the scan turns
+//       into the workgroups' starts), then route and group bases [2][257].
 // ---------------------------------------------------------------------------------------------
 constexpr uint32_t kWideRoutesPerWave = 256, kWideRoutesPerGroup = kPlanWaves * kWideRoutesPerWave;
 __host__ __device__ constexpr uint32_t wide_plan_groups(uint32_t routes) { return (routes + kWideRoutesPerGroup - 1) / kWideRoutesPerGroup; }
 __host__ __device__ constexpr uint64_t wide_plan_words(uint32_t routes) {
-    return 4 + uint64_t(wide_plan_groups(routes)) * kPlanWaves * 256 + 2 * 257;
+    return 4 + uint64_t(wide_plan_groups(routes)) * (kPlanWaves + 1) * 256 + 2 * 257;
 }
 
 __global__ void __launch_bounds__(kPlanThreads)
@@ -382,14 +387,22 @@ plan_count_kernel(const int32_t* __restrict__ ids, const float* __restrict__ w, 
             if (!below) hist[wv][e] += __popcll(m);
         }
     }
-    uint32_t* mine = work + 4 + (uint64_t(blockIdx.x) * kPlanWaves + wv) * 256;
+    __syncthreads();
+    if (tid < 256) {  // per expert: every wave's start inside this workgroup, and the workgroup's total
+        uint32_t* starts = work + 4 + uint64_t(blockIdx.x) * kPlanWaves * 256 + tid;
+        uint32_t run = 0;
 #pragma unroll
-    for (uint32_t j = 0; j < 4; ++j) mine[lane + 64 * j] = hist[wv][lane + 64 * j];  // the wave's own row: no barrier needed
+        for (uint32_t k = 0; k < kPlanWaves; ++k) {
+            starts[k * 256] = run;
+            run += hist[k][tid];
+        }
+        work[4 + uint64_t(gridDim.x) * kPlanWaves * 256 + blockIdx.x * 256 + tid] = run;
+    }
 }
 
 __global__ void __launch_bounds__(kPlanThreads)
 plan_scan_kernel(uint32_t routes, uint32_t* __restrict__ work, PlanView p, uint32_t gpc) {
-    __shared__ uint32_t part[4][256], cnt[256], rbase[257], gbase[257], cbase[257];
+    __shared__ uint32_t cnt[256], rbase[257], gbase[257], cbase[257];
     const uint32_t tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
     const uint32_t waves = wide_plan_groups(routes) * kPlanWaves;
     const uint32_t first_bad = work[0];
@@ -403,24 +416,21 @@ plan_scan_kernel(uint32_t routes, uint32_t* __restrict__ work, PlanView p, uint3
         }
         return;
     }
-    // Four threads per expert each total a quarter of the waves, then turn the counts of their
-    // quarter into running starts.
-    uint32_t* counts = work + 4;
-    const uint32_t e = tid & 255, quarter = tid >> 8, per = (waves + 3) / 4;
-    const uint32_t k0 = quarter * per, k1 = k0 + per < waves ? k0 + per : waves;
-    uint32_t sum = 0;
-#pragma unroll 16
-    for (uint32_t k = k0; k < k1; ++k) sum += counts[uint64_t(k) * 256 + e];  // unrolled: the loads are independent, the walk is latency
-    part[quarter][e] = sum;
-    __syncthreads();
-    uint32_t run = 0;
-    for (uint32_t qd = 0; qd < quarter; ++qd) run += part[qd][e];
-    if (quarter == 3) cnt[e] = run + sum;
-#pragma unroll 16
-    for (uint32_t k = k0; k < k1; ++k) {
-        const uint32_t c = counts[uint64_t(k) * 256 + e];
-        counts[uint64_t(k) * 256 + e] = run;
-        run += c;
+    // One thread per expert turns the workgroups' totals into the workgroups' starts (all loads first: the walk
+    // is latency) and leaves the expert's row count.
+    const uint32_t groups = wide_plan_groups(routes);
+    uint32_t* totals = work + 4 + uint64_t(waves) * 256;
+    if (tid < 256) {
+        uint32_t t[kMaxRows * kTopk / kWideRoutesPerGroup];
+#pragma unroll
+        for (uint32_t g = 0; g < kMaxRows * kTopk / kWideRoutesPerGroup; ++g) t[g] = g < groups ? totals[g * 256 + tid] : 0;
+        uint32_t run = 0;
+#pragma unroll
+        for (uint32_t g = 0; g < kMaxRows * kTopk / kWideRoutesPerGroup; ++g) {
+            if (g < groups) totals[g * 256 + tid] = run;
+            run += t[g];
+        }
+        cnt[tid] = run;
     }
     __syncthreads();
     if (wv == 0) {
@@ -436,7 +446,7 @@ plan_scan_kernel(uint32_t routes, uint32_t* __restrict__ work, PlanView p, uint3
         wave_scan256(c, cbase, lane);
     }
     __syncthreads();
-    uint32_t* bases = work + 4 + uint64_t(waves) * 256;
+    uint32_t* bases = work + 4 + uint64_t(waves + groups) * 256;
     for (uint32_t i = tid; i < 257; i += kPlanThreads) {
         bases[i] = rbase[i];
         bases[257 + i] = gbase[i];
@@ -471,10 +481,11 @@ plan_place_kernel(const int32_t* __restrict__ ids, const float* __restrict__ w, 
     if (p.meta[kPlanFault]) return;  // a rejected plan writes nothing
     const uint32_t tid = threadIdx.x, lane = tid & 63, wv = tid >> 6, routes = rows * kTopk;
     const uint32_t waves = wide_plan_groups(routes) * kPlanWaves;
-    const uint32_t* mine = work + 4 + (uint64_t(blockIdx.x) * kPlanWaves + wv) * 256;
-    const uint32_t* bases = work + 4 + uint64_t(waves) * 256;
+    const uint32_t* mine = work + 4 + (uint64_t(blockIdx.x) * kPlanWaves + wv) * 256;   // the wave's starts inside this workgroup
+    const uint32_t* ours = work + 4 + uint64_t(waves) * 256 + blockIdx.x * 256;          // this workgroup's starts
+    const uint32_t* bases = work + 4 + uint64_t(waves + gridDim.x) * 256;
 #pragma unroll
-    for (uint32_t j = 0; j < 4; ++j) start[wv][lane + 64 * j] = mine[lane + 64 * j];
+    for (uint32_t j = 0; j < 4; ++j) start[wv][lane + 64 * j] = mine[lane + 64 * j] + ours[lane + 64 * j];
     for (uint32_t i = tid; i < 257; i += kPlanThreads) {
         rbase[i] = bases[i];
         gbase[i] = bases[257 + i];
