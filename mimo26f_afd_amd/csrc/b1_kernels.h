@@ -8,7 +8,10 @@
 //   fc1_kernel      <- kernels/b1/grouped.cu:74-113 + connected.cu:9-37 (gate/up MMA + SwiGLU)
 //                      fused with kernels/b1/quant_v1.cu:34-68 (intermediate quantizer v1)
 //   fc2_kernel      <- kernels/b1/grouped.cu:135-154 + connected.cu:48-79 (down MMA + inverse scatter)
-//   reduce_kernel   <- kernels/b1/route_reduce.cu:61-124 (weight-once slot-ordered sum, BF16 RNE)
+//   reduce_kernel   <- kernels/b1/route_reduce.cu:61-124 (weight-once slot-ordered sum, BF16 RNE); the same
+//                      arithmetic (combine4) runs inside the FC2 kernels when the combine is fused
+//                      (combine_completed), and on BF16 per-route rows in the opt-in mode of
+//                      crates/mimo26-spark/kernels/b1_serve.cu:98-143
 //   quantize_kernel <- kernels/b1/quant_v1.cu:34-68 (stand-alone form, same device functions)
 #pragma once
 #include <hip/hip_runtime.h>
