@@ -863,7 +863,8 @@ __device__ __forceinline__ ItemHead load_item_head(const Chunk* record, const ui
 }
 
 // Stages 2+3: gate/up grouped GEMM, SwiGLU and the v1 requantisation of the intermediate.
-// grid (I/128, chunk capacity), 256 threads; each wave owns one 32-column K32 block of the
+// grid (I/128, chunk capacity) x 256 threads, or (I/32, chunk capacity) x 64 for the smallest calls (the waves
+// share nothing; the host picks the workgroup); each wave owns one 32-column K32 block of the
 // intermediate for every row of its chunk, so a quantizer block never leaves the wave. A chunk
 // holds at most NT groups; the body is compiled for 1, 2, 4 and 8 activation tiles.
 template <int NT>
@@ -873,7 +874,7 @@ __global__ void __launch_bounds__(256) fc1_kernel(Fc1Args a) {
     const ItemHead head = load_item_head(a.plan.chunks + c, meta);  // the chunk table covers the whole grid
     const Chunk ch = head.ch;
     if (head.meta[kPlanFault] || c >= head.meta[kChunkCount]) return;
-    const uint32_t lane = threadIdx.x & 63, cb = blockIdx.x * 4 + (threadIdx.x >> 6);
+    const uint32_t lane = threadIdx.x & 63, cb = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
     const int32_t expert = ch.expert;
     if (expert < 0 || expert >= int32_t(kExperts) || ch.groups < 1 || ch.groups > NT) {
         if (lane == 0) atomicOr(&meta[kFc1Fault], 2u);
@@ -1095,7 +1096,7 @@ __device__ __forceinline__ void fc2_body(const Fc2Args& a, const Chunk ch, uint3
 }
 
 // Stage 4a: down grouped GEMM on the requantised intermediate; rows go back to y[original route].
-// grid (16, chunk capacity), 256 threads; each wave owns 64 output columns. (Two neighbouring blocks per wave
+// grid (16, chunk capacity) x 256 threads or (64, chunk capacity) x 64; each wave owns 64 output columns. (Two neighbouring blocks per wave
 // in one stream halve the workgroups, and at 128 tokens the longer tail of the launch cost more than the longer
 // streams saved, 172 against 154 us.)
 template <int NT>
@@ -1105,7 +1106,7 @@ __global__ void __launch_bounds__(256) fc2_kernel(Fc2Args a) {
     const ItemHead head = load_item_head(a.plan.chunks + c, meta);
     const Chunk ch = head.ch;
     if (head.meta[kPlanFault] || head.meta[kFc1Fault] || head.meta[kQuantFault] || c >= head.meta[kChunkCount]) return;
-    const uint32_t lane = threadIdx.x & 63, ob = blockIdx.x * 4 + (threadIdx.x >> 6);
+    const uint32_t lane = threadIdx.x & 63, ob = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
     const int32_t expert = ch.expert;
     if (expert < 0 || expert >= int32_t(kExperts) || ch.groups < 1 || ch.groups > NT) {
         if (lane == 0) atomicOr(&meta[kFc2Fault], 2u);
