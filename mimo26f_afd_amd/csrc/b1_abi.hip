@@ -350,14 +350,16 @@ Fc2Args fc2_args(const m26s_b1_layer* L, const Launch& k, const float* w, uint16
 }
 
 // Decode-size calls: every wave streams its own weight block from HBM, activations from L2.
-// The waves of these kernels share nothing, so the workgroup is only the unit the dispatcher hands out. Up to
-// 48 tokens a launch is a few rounds of workgroups at most, and one-wave workgroups fill the compute units
-// evenly where four-wave ones leave the last round part empty (8 tokens: 58.7 against 64.2 us per call, 16:
-// 95.6 against 102.4, 32: 168 against 171); from 96 tokens on the four-wave form is the faster by half a percent.
-constexpr uint64_t kNarrowRoutes = 48 * kTopk;
+// The waves of these kernels share nothing, so the workgroup is only the unit the dispatcher hands out. Below
+// 32 tokens a launch is a round or two of workgroups, and one-wave workgroups fill the compute units evenly
+// where four-wave ones leave the last round part empty (per call, one wave against four: 8 tokens 58.7 / 64.2 us,
+// 16 tokens 95.6 / 102.4, 24 tokens 130 / 134; one expert's 16 rows at a rank's share 36.8 / 41.6). At 32 tokens
+// the two are within 1 % of each other either way (full intermediate 168 / 171, 256 experts of a rank's share with
+// one row each 136.2 / 135.1), and from 96 tokens on the four-wave form is the faster by half a percent.
+constexpr uint64_t kNarrowRoutes = 32 * kTopk;
 template <int NT>
 void launch_direct(const m26s_b1_layer* L, const Launch& k, const Fc1Args& f1, const Fc2Args& f2) {
-    const uint32_t waves = k.ws.routes <= kNarrowRoutes ? 1 : 4;
+    const uint32_t waves = k.ws.routes < kNarrowRoutes ? 1 : 4;
     fc1_kernel<NT><<<dim3(L->lay.inter / (32 * waves), k.ws.chunk_cap), 64 * waves, 0, k.stream>>>(f1);
     mark(k.fc1_done, k.stream);
     fc2_kernel<NT><<<dim3(kHidden / (64 * waves), k.ws.chunk_cap), 64 * waves, 0, k.stream>>>(f2);
