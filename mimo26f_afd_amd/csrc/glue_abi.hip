@@ -16,6 +16,24 @@ int grid_for(long n) {
 
 int launched() { return int(hipGetLastError()); }
 
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+// Launch shape of quantize_hidden_kernel: 32 blocks of a row per workgroup along x, rows along y, two rows per
+// thread and step. Rows whose outputs are contiguous are one long row to the kernel (x always is).
+int launch_quantize(const float* x, long rows, long per_row, uint8_t* payload, size_t payload_pitch, uint8_t* scales,
+                    size_t scales_pitch, float* scale_inv, void* stream) {
+    const bool flat = (!payload || payload_pitch == size_t(per_row) * 32) && scales_pitch == size_t(per_row);
+    if (flat) {
+        per_row *= rows;
+        rows = 1;
+    }
+    const long pieces = (per_row + 31) / 32, lines = (rows + 1) / 2;
+    if (pieces > 0x7fffffffL) return 1;
+    quantize_hidden_kernel<<<dim3(unsigned(pieces), unsigned(lines < 4096 ? lines : 4096)), kThreads, 0, hipStream_t(stream)>>>(
+        x, rows, per_row, payload, payload_pitch, scales, scales_pitch, scale_inv);
+    return launched();
+}
+
 }  // namespace
 
 extern "C" {
@@ -34,9 +52,7 @@ int m26c_router_topk(const float* logits, const float* bias, int rows, int n_exp
 int m26c_quant_scales(const float* x, long n_blocks, unsigned char* scales, float* scale_inv, void* stream) {
     if (n_blocks <= 0) return 0;
     if (!x || !scales || !scale_inv) return 1;
-    quantize_hidden_kernel<<<grid_for(n_blocks * 8), kThreads, 0, hipStream_t(stream)>>>(x, n_blocks, 32, nullptr, 0, scales, 1,
-                                                                                        scale_inv);
-    return launched();
+    return launch_quantize(x, n_blocks, 1, nullptr, 0, scales, 1, scale_inv, stream);
 }
 
 int m26_quantize_hidden_fp8(const float* x, const float* scale_inv, uint8_t* payload, int64_t n_elem, void* stream) {
@@ -52,9 +68,7 @@ int m26c_quantize_hidden(const float* x, long rows, int cols, uint8_t* payload, 
     if (!x || !payload || !scales || cols <= 0 || cols % 32 || payload_pitch < size_t(cols) || scales_pitch < size_t(cols / 32) ||
         payload_pitch % 4)
         return 1;
-    quantize_hidden_kernel<<<grid_for(rows * (cols / 32) * 8), kThreads, 0, hipStream_t(stream)>>>(
-        x, rows, cols, payload, payload_pitch, scales, scales_pitch, nullptr);
-    return launched();
+    return launch_quantize(x, rows, cols / 32, payload, payload_pitch, scales, scales_pitch, nullptr, stream);
 }
 
 int m26c_frame_fill(const int* idx, const float* wts, const uint8_t* payload, const uint8_t* scales, int t, int topk,
@@ -77,21 +91,30 @@ int m26c_rank_sum_bf16(const uint16_t* p0, const uint16_t* p1, const uint16_t* p
                        long n, void* stream) {
     if (n <= 0) return 0;
     if (!p0 || !p1 || !p2 || !p3 || !out) return 1;
-    rank_sum_bf16_kernel<<<grid_for(n), kThreads, 0, hipStream_t(stream)>>>(p0, p1, p2, p3, out, n);
+    if (aligned16(p0) && aligned16(p1) && aligned16(p2) && aligned16(p3) && aligned16(out))
+        rank_sum_bf16_kernel<true><<<grid_for((n + 7) / 8), kThreads, 0, hipStream_t(stream)>>>(p0, p1, p2, p3, out, n);
+    else
+        rank_sum_bf16_kernel<false><<<grid_for(n), kThreads, 0, hipStream_t(stream)>>>(p0, p1, p2, p3, out, n);
     return launched();
 }
 
 int m26c_add_inplace(float* h, const float* a, long n, void* stream) {
     if (n <= 0) return 0;
     if (!h || !a) return 1;
-    add_inplace_kernel<<<grid_for(n), kThreads, 0, hipStream_t(stream)>>>(h, a, n);
+    if (aligned16(h) && aligned16(a))
+        add_inplace_kernel<true><<<grid_for((n + 7) / 8), kThreads, 0, hipStream_t(stream)>>>(h, a, n);
+    else
+        add_inplace_kernel<false><<<grid_for(n), kThreads, 0, hipStream_t(stream)>>>(h, a, n);
     return launched();
 }
 
 int m26c_f32_to_bf16(const float* x, uint16_t* y, long n, void* stream) {
     if (n <= 0) return 0;
     if (!x || !y) return 1;
-    f32_to_bf16_kernel<<<grid_for(n), kThreads, 0, hipStream_t(stream)>>>(x, y, n);
+    if (aligned16(x) && aligned16(y))
+        f32_to_bf16_kernel<true><<<grid_for((n + 7) / 8), kThreads, 0, hipStream_t(stream)>>>(x, y, n);
+    else
+        f32_to_bf16_kernel<false><<<grid_for(n), kThreads, 0, hipStream_t(stream)>>>(x, y, n);
     return launched();
 }
 

@@ -89,63 +89,62 @@ __device__ __forceinline__ uint32_t q0_scale_byte(float amax) {
 // E4M3FN code nearest to y = x * scale (scale a positive power of two), ties to the larger magnitude,
 // saturating at 448, NaN -> 0. The sign bit is "the exact product is below zero", i.e. x < 0: -0.0
 // gives 0x00 while a negative value that rounds to zero keeps 0x80, also where the binary32 product
-// has already underflowed to -0 (the CPU rule multiplies in binary64). Integer arithmetic on the
-// significand: round-half-up is an add and a shift.
+// has already underflowed to -0 (the CPU rule multiplies in binary64). Integer arithmetic on the bit
+// pattern: from 2^-6 up a code is the binary32 exponent and top three mantissa bits rebased, so
+// round-half-up is one add and one shift and a mantissa that rounds over carries into the exponent by
+// itself (448, the clamp, is code 0x7e exactly, so nothing larger can come out); below 2^-6 the
+// quantum is 2^-9 whatever the exponent, and the significand is shifted down to it.
 __device__ __forceinline__ uint32_t e4m3_half_up(float x, float scale) {
     const float y = x * scale;
-    if (y != y) return 0;
     const uint32_t sign = x < 0.0f ? 0x80u : 0u;
-    float mag = fabsf(y);
-    mag = mag > 448.0f ? 448.0f : mag;
-    const uint32_t bits = __float_as_uint(mag), field = bits >> 23;
-    if (field < 127 - 11) return sign;  // below 2^-11: under half the smallest step (zero and subnormals too)
-    const int e = int(field) - 127;
-    const uint32_t sig = (bits & 0x7fffffu) | 0x800000u;  // value = sig * 2^(e - 23)
-    if (e < -6) {                                          // quantum 2^-9: code = floor(value * 512 + 1/2)
-        const int sh = 14 - e;                             // >= 21
-        return sign | ((sig + (1u << (sh - 1))) >> sh);    // 8 is the smallest normal code
+    const float mag = fminf(fabsf(y), 448.0f);             // a NaN leaves here as 448 and is zeroed at the end
+    const uint32_t bits = __float_as_uint(mag);
+    uint32_t code = ((bits + 0x80000u) >> 20) - ((127u - 7u) << 3);
+    if (bits < (121u << 23)) {                              // below 2^-6: code = floor(value * 512 + 1/2)
+        const uint32_t sig = (bits & 0x7fffffu) | 0x800000u, sh = 141u - (bits >> 23);  // value = sig * 2^(field - 150); sh >= 21
+        code = sh > 31u ? 0u : (sig + (1u << (sh - 1u))) >> sh;  // under 2^-11 (zero and binary32 subnormals too): nothing
     }
-    uint32_t q = (sig + 0x80000u) >> 20;                   // 8 .. 16
-    uint32_t ee = uint32_t(e + 7);
-    if (q == 16) { q = 8; ++ee; }
-    const uint32_t code = (ee << 3) | (q - 8);
-    return sign | (code > 0x7eu ? 0x7eu : code);
+    return y != y ? 0u : sign | code;
 }
 
-// One K32 block per 8 lanes, four values per lane. grid-stride over blocks.
-__global__ void __launch_bounds__(256) quantize_hidden_kernel(const float* __restrict__ x, long rows, int cols,
+// One K32 block per 8 lanes, four values per lane; a workgroup takes 32 consecutive blocks of a row
+// (1024 values), blockIdx.x choosing the piece of the row and blockIdx.y striding over rows, so no
+// thread divides anything. x is contiguous (row r starts at r * 32 * per_row); payload and scales
+// have their own pitches. Two rows are in flight per thread and step.
+__global__ void __launch_bounds__(256) quantize_hidden_kernel(const float* __restrict__ x, long rows, long per_row,
                                                               uint8_t* __restrict__ payload, size_t payload_pitch,
                                                               uint8_t* __restrict__ scales, size_t scales_pitch,
                                                               float* __restrict__ scale_inv) {
-    const int sub = threadIdx.x & 7, per_row = cols / 32;
-    const long blocks = rows * per_row;
-    const long stride = (long(gridDim.x) * blockDim.x) >> 3;
-    // Whole waves walk together: the shuffles below need all eight lanes of a block present.
-    const long first = (long(blockIdx.x) * blockDim.x + threadIdx.x) >> 3;
-    const long rounds = (blocks + stride - 1) / stride;
-    for (long it = 0; it < rounds; ++it) {
-        const long b = first + it * stride;
-        const bool live = b < blocks;
-        const long r = live ? b / per_row : 0, c = live ? b % per_row : 0;
-        float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (live) v = *reinterpret_cast<const float4*>(x + (r * cols + c * 32 + sub * 4));
-        // NaNs take no part in amax. They are zeroed first: a signalling NaN would come out of the
-        // hardware maximum as a quiet one and wipe what was gathered before it.
-        auto mag = [](float f) { return f != f ? 0.0f : fabsf(f); };
+    const uint32_t sub = threadIdx.x & 7;
+    const long c = long(blockIdx.x) * 32 + (threadIdx.x >> 3);
+    const bool in_row = c < per_row;  // the same for all eight lanes of a block, so the shuffles below see whole blocks
+    // NaNs take no part in amax. They are zeroed first: a signalling NaN would come out of the
+    // hardware maximum as a quiet one and wipe what was gathered before it.
+    auto mag = [](float f) { return f != f ? 0.0f : fabsf(f); };
+    auto finish = [&](long r, const float4 v) {
         float amax = fmaxf(fmaxf(mag(v.x), mag(v.y)), fmaxf(mag(v.z), mag(v.w)));
 #pragma unroll
         for (int d = 4; d; d >>= 1) amax = fmaxf(amax, __shfl_xor(amax, d));
         const uint32_t s = q0_scale_byte(amax);
         // 2^(127 - s): exponent field 254 - s; s = 254 is 2^-127, the subnormal with the top mantissa bit
         const float scale = __uint_as_float(s == 254u ? 0x00400000u : (254u - s) << 23);
-        if (!live) continue;
-        const uint32_t word = e4m3_half_up(v.x, scale) | e4m3_half_up(v.y, scale) << 8 | e4m3_half_up(v.z, scale) << 16 |
-                              e4m3_half_up(v.w, scale) << 24;
-        if (payload) *reinterpret_cast<uint32_t*>(payload + r * payload_pitch + c * 32 + sub * 4) = word;
+        if (!in_row) return;
+        if (payload)
+            *reinterpret_cast<uint32_t*>(payload + r * payload_pitch + c * 32 + sub * 4) =
+                e4m3_half_up(v.x, scale) | e4m3_half_up(v.y, scale) << 8 | e4m3_half_up(v.z, scale) << 16 | e4m3_half_up(v.w, scale) << 24;
         if (sub == 0) {
             if (scales) scales[r * scales_pitch + c] = uint8_t(s);
-            if (scale_inv) scale_inv[b] = scale;
+            if (scale_inv) scale_inv[r * per_row + c] = scale;
         }
+    };
+    const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
+    const long step = gridDim.y;
+    for (long r = blockIdx.y; r < rows; r += 2 * step) {  // uniform over the workgroup
+        const long r2 = r + step;
+        const float4 v = in_row ? *reinterpret_cast<const float4*>(x + ((r * per_row + c) * 32 + sub * 4)) : zero;
+        const float4 v2 = in_row && r2 < rows ? *reinterpret_cast<const float4*>(x + ((r2 * per_row + c) * 32 + sub * 4)) : zero;
+        finish(r, v);
+        if (r2 < rows) finish(r2, v2);
     }
 }
 
@@ -204,31 +203,80 @@ __global__ void __launch_bounds__(256) frame_fill_kernel(const int* __restrict__
 // ---- rank sum, residual, BF16 cast -----------------------------------------------------------------
 __device__ __forceinline__ float bf16_value(uint32_t bits) { return __uint_as_float(bits << 16); }
 
+// The three kernels below move eight values per lane and step in 16-byte accesses when every pointer is
+// 16-byte aligned (VEC; the host checks), one value per lane otherwise; the last n % 8 values are taken one
+// by one by the first lanes of the grid.
+template <typename F>
+__device__ __forceinline__ void each_eight(long n, F&& body8, bool vec) {
+    const long tid = long(blockIdx.x) * blockDim.x + threadIdx.x, threads = long(gridDim.x) * blockDim.x;
+    const long groups = vec ? n / 8 : 0;
+    for (long g = tid; g < groups; g += threads) body8(g * 8, true);
+    for (long i = groups * 8 + tid; i < n; i += threads) body8(i, false);
+}
+
 // s = 0; s += rank 0, 1, 2, 3: four separate FP32 additions, in that order.
+__device__ __forceinline__ float rank_sum4(uint32_t a, uint32_t b, uint32_t c, uint32_t d) {
+    float s = 0.0f;
+    s = __fadd_rn(s, bf16_value(a));
+    s = __fadd_rn(s, bf16_value(b));
+    s = __fadd_rn(s, bf16_value(c));
+    return __fadd_rn(s, bf16_value(d));
+}
+template <bool VEC>
 __global__ void __launch_bounds__(256) rank_sum_bf16_kernel(const uint16_t* __restrict__ p0, const uint16_t* __restrict__ p1,
                                                             const uint16_t* __restrict__ p2, const uint16_t* __restrict__ p3,
                                                             float* __restrict__ out, long n) {
-    for (long i = long(blockIdx.x) * blockDim.x + threadIdx.x; i < n; i += long(gridDim.x) * blockDim.x) {
-        float s = 0.0f;
-        s = __fadd_rn(s, bf16_value(p0[i]));
-        s = __fadd_rn(s, bf16_value(p1[i]));
-        s = __fadd_rn(s, bf16_value(p2[i]));
-        s = __fadd_rn(s, bf16_value(p3[i]));
-        out[i] = s;
-    }
+    each_eight(n, [&](long i, bool eight) {
+        if (!eight) {
+            out[i] = rank_sum4(p0[i], p1[i], p2[i], p3[i]);
+            return;
+        }
+        const uint4 a = *reinterpret_cast<const uint4*>(p0 + i), b = *reinterpret_cast<const uint4*>(p1 + i),
+                    c = *reinterpret_cast<const uint4*>(p2 + i), d = *reinterpret_cast<const uint4*>(p3 + i);
+        const uint32_t wa[4] = {a.x, a.y, a.z, a.w}, wb[4] = {b.x, b.y, b.z, b.w}, wc[4] = {c.x, c.y, c.z, c.w}, wd[4] = {d.x, d.y, d.z, d.w};
+        float o[8];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {  // a dword holds two values, the lower address in the low half
+            o[2 * j] = rank_sum4(wa[j] & 0xffffu, wb[j] & 0xffffu, wc[j] & 0xffffu, wd[j] & 0xffffu);
+            o[2 * j + 1] = rank_sum4(wa[j] >> 16, wb[j] >> 16, wc[j] >> 16, wd[j] >> 16);
+        }
+        *reinterpret_cast<float4*>(out + i) = make_float4(o[0], o[1], o[2], o[3]);
+        *reinterpret_cast<float4*>(out + i + 4) = make_float4(o[4], o[5], o[6], o[7]);
+    }, VEC);
 }
 
+template <bool VEC>
 __global__ void __launch_bounds__(256) add_inplace_kernel(float* __restrict__ h, const float* __restrict__ a, long n) {
-    for (long i = long(blockIdx.x) * blockDim.x + threadIdx.x; i < n; i += long(gridDim.x) * blockDim.x)
-        h[i] = __fadd_rn(h[i], a[i]);
+    each_eight(n, [&](long i, bool eight) {
+        if (!eight) {
+            h[i] = __fadd_rn(h[i], a[i]);
+            return;
+        }
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const float4 u = *reinterpret_cast<const float4*>(h + i + 4 * j), v = *reinterpret_cast<const float4*>(a + i + 4 * j);
+            *reinterpret_cast<float4*>(h + i + 4 * j) =
+                make_float4(__fadd_rn(u.x, v.x), __fadd_rn(u.y, v.y), __fadd_rn(u.z, v.z), __fadd_rn(u.w, v.w));
+        }
+    }, VEC);
 }
 
 // Round to nearest even; a NaN becomes 0x7fff, as the reference's conversion intrinsic gives.
+__device__ __forceinline__ uint32_t bf16_rne_nan(float f) {
+    const uint32_t b = __float_as_uint(f);
+    return (b & 0x7fffffffu) > 0x7f800000u ? 0x7fffu : (b + 0x7fffu + ((b >> 16) & 1u)) >> 16;
+}
+template <bool VEC>
 __global__ void __launch_bounds__(256) f32_to_bf16_kernel(const float* __restrict__ x, uint16_t* __restrict__ y, long n) {
-    for (long i = long(blockIdx.x) * blockDim.x + threadIdx.x; i < n; i += long(gridDim.x) * blockDim.x) {
-        const uint32_t b = __float_as_uint(x[i]);
-        y[i] = (b & 0x7fffffffu) > 0x7f800000u ? uint16_t(0x7fff) : uint16_t((b + 0x7fffu + ((b >> 16) & 1u)) >> 16);
-    }
+    each_eight(n, [&](long i, bool eight) {
+        if (!eight) {
+            y[i] = uint16_t(bf16_rne_nan(x[i]));
+            return;
+        }
+        const float4 u = *reinterpret_cast<const float4*>(x + i), v = *reinterpret_cast<const float4*>(x + i + 4);
+        *reinterpret_cast<uint4*>(y + i) = make_uint4(bf16_rne_nan(u.x) | bf16_rne_nan(u.y) << 16, bf16_rne_nan(u.z) | bf16_rne_nan(u.w) << 16,
+                                                      bf16_rne_nan(v.x) | bf16_rne_nan(v.y) << 16, bf16_rne_nan(v.z) | bf16_rne_nan(v.w) << 16);
+    }, VEC);
 }
 
 }  // namespace m26g

@@ -124,6 +124,48 @@ def test_rank_sum_residual_and_cast_bit_exact():
     assert np.array_equal(y.to_host(np.uint16), O.bf16_rne_nan(x))
 
 
+def test_elementwise_kernels_on_unaligned_pointers_and_short_arrays():
+    """The 16-byte forms need 16-byte aligned pointers; anything else takes the one-value form. Same bits either
+    way, for every length from none to a few groups of eight."""
+    rng = np.random.default_rng(12)
+    for n in (1, 7, 8, 9, 23, 4099):
+        for shift in (0, 1, 2):                                  # in elements: 0 keeps the device buffer's alignment
+            p = (rng.standard_normal((4, n + shift)) * 8).astype(np.float32)
+            bits = (p.view(np.uint32) >> 16).astype(np.uint16)
+            planes, out = [dev(b) for b in bits], D((n + shift) * 4)
+            glue.rank_sum_bf16(*[b.ptr + 2 * shift for b in planes], out.ptr + 4 * shift, n)
+            got = out.to_host(np.float32)[shift:shift + n]
+            assert np.array_equal(got.view(np.uint32), O.rank_sum_bf16(*bits[:, shift:]).view(np.uint32)), (n, shift)
+            h = rng.standard_normal(n + shift).astype(np.float32)
+            dh = dev(h)
+            glue.add_inplace(dh.ptr + 4 * shift, out.ptr + 4 * shift, n)
+            back = dh.to_host(np.float32)
+            assert np.array_equal(back[shift:].view(np.uint32), (h[shift:] + got).astype(np.float32).view(np.uint32)), (n, shift)
+            assert np.array_equal(back[:shift], h[:shift])
+            y = D((n + shift) * 2)
+            glue.f32_to_bf16(dh.ptr + 4 * shift, y.ptr + 2 * shift, n)
+            assert np.array_equal(y.to_host(np.uint16)[shift:shift + n], O.bf16_rne_nan(back[shift:])), (n, shift)
+
+
+def test_wire_quantizer_row_shapes():
+    """Rows shorter than a workgroup's 1024 values, rows that are not a multiple of it, and pitched outputs: the
+    same bytes as the CPU rule row by row."""
+    rng = np.random.default_rng(13)
+    for rows, cols, ppitch, spitch in ((5, 32, 32, 1), (3, 96, 96, 3), (7, 1056, 1056, 33), (4, 1056, 1088, 40), (9, 4096, 4224, 4224),
+                                       (1, 4096, 4096, 128), (6, 64, 80, 2)):
+        x = synth.bf16_round((rng.standard_normal((rows, cols)) * np.exp2(rng.integers(-20, 20, (rows, 1)))).astype(np.float32))
+        ref_p, ref_s = O.q0_quantize(x)
+        in_frame = spitch == ppitch and ppitch > cols           # scales behind the payload of the same row
+        dp = D(rows * ppitch + 64)
+        dsc = dp if in_frame else D(rows * spitch + 64)
+        glue.quantize_hidden(dev(x).ptr, rows, cols, dp.ptr, ppitch, dsc.ptr + (cols if in_frame else 0), spitch)
+        got_p = dp.to_host(np.uint8)[: rows * ppitch].reshape(rows, ppitch)[:, :cols]
+        raw_s = dsc.to_host(np.uint8)
+        got_s = (raw_s[cols: cols + rows * spitch] if in_frame else raw_s[: rows * spitch])
+        got_s = np.lib.stride_tricks.as_strided(got_s, (rows, cols // 32), (spitch, 1))
+        assert np.array_equal(got_p, ref_p) and np.array_equal(got_s, ref_s), (rows, cols, ppitch, spitch)
+
+
 def test_chain_router_quantizer_frame_ffn():
     """FP32 logits and bf16-valued hidden rows in; the GPU routes, quantizes into a request frame and the
     FFN reads the frame rows in place: the same BF16 bits as the FFN fed with the checker's bytes."""
