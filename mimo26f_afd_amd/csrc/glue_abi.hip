@@ -18,19 +18,25 @@ int launched() { return int(hipGetLastError()); }
 
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
-// Launch shape of quantize_hidden_kernel: 32 blocks of a row per workgroup along x, rows along y, two rows per
-// thread and step. Rows whose outputs are contiguous are one long row to the kernel (x always is).
+// Launch shape of quantize_hidden_kernel: 32 blocks of a row per workgroup along x, rows along y, four rows per
+// thread and step. Rows whose outputs are contiguous are one long array (x always is), cut into rows of 32
+// blocks so that every thread still has its four loads in flight.
 int launch_quantize(const float* x, long rows, long per_row, uint8_t* payload, size_t payload_pitch, uint8_t* scales,
                     size_t scales_pitch, float* scale_inv, void* stream) {
-    const bool flat = (!payload || payload_pitch == size_t(per_row) * 32) && scales_pitch == size_t(per_row);
-    if (flat) {
-        per_row *= rows;
-        rows = 1;
+    const long total = rows * per_row;
+    if ((!payload || payload_pitch == size_t(per_row) * 32) && scales_pitch == size_t(per_row)) {
+        per_row = 32;
+        rows = (total + 31) / 32;
+        payload_pitch = 1024;
+        scales_pitch = 32;
     }
-    const long pieces = (per_row + 31) / 32, lines = (rows + 1) / 2;
+    // About four workgroups per compute unit, each walking several sets of rows with the next set's loads in flight.
+    const long pieces = (per_row + 31) / 32, lines = (rows + kQuantRowsInFlight - 1) / kQuantRowsInFlight;
     if (pieces > 0x7fffffffL) return 1;
-    quantize_hidden_kernel<<<dim3(unsigned(pieces), unsigned(lines < 4096 ? lines : 4096)), kThreads, 0, hipStream_t(stream)>>>(
-        x, rows, per_row, payload, payload_pitch, scales, scales_pitch, scale_inv);
+    long walkers = pieces >= 1024 ? 1 : 1024 / pieces;
+    walkers = walkers < lines ? walkers : lines;
+    quantize_hidden_kernel<<<dim3(unsigned(pieces), unsigned(walkers)), kThreads, 0, hipStream_t(stream)>>>(
+        x, rows, per_row, total, payload, payload_pitch, scales, scales_pitch, scale_inv);
     return launched();
 }
 

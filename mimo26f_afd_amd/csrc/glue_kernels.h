@@ -94,57 +94,139 @@ __device__ __forceinline__ uint32_t q0_scale_byte(float amax) {
 // round-half-up is one add and one shift and a mantissa that rounds over carries into the exponent by
 // itself (448, the clamp, is code 0x7e exactly, so nothing larger can come out); below 2^-6 the
 // quantum is 2^-9 whatever the exponent, and the significand is shifted down to it.
+constexpr uint32_t kE4m3NormalFrom = 121u << 23;  // binary32 bits of 2^-6
+__device__ __forceinline__ uint32_t e4m3_magnitude_bits(float y) { return __float_as_uint(fminf(fabsf(y), 448.0f)); }  // a NaN leaves as 448
+__device__ __forceinline__ uint32_t e4m3_code_normal(uint32_t bits) { return ((bits + 0x80000u) >> 20) - ((127u - 7u) << 3); }
+__device__ __forceinline__ uint32_t e4m3_code_small(uint32_t bits) {  // code = floor(value * 512 + 1/2)
+    const uint32_t sig = (bits & 0x7fffffu) | 0x800000u, sh = 141u - (bits >> 23);  // value = sig * 2^(field - 150); sh >= 21
+    return sh > 31u ? 0u : (sig + (1u << (sh - 1u))) >> sh;  // under 2^-11 (zero and binary32 subnormals too): nothing
+}
+__device__ __forceinline__ uint32_t e4m3_signed(float x, float y, uint32_t code) {
+    return y != y ? 0u : (x < 0.0f ? 0x80u : 0u) | code;
+}
 __device__ __forceinline__ uint32_t e4m3_half_up(float x, float scale) {
     const float y = x * scale;
-    const uint32_t sign = x < 0.0f ? 0x80u : 0u;
-    const float mag = fminf(fabsf(y), 448.0f);             // a NaN leaves here as 448 and is zeroed at the end
-    const uint32_t bits = __float_as_uint(mag);
-    uint32_t code = ((bits + 0x80000u) >> 20) - ((127u - 7u) << 3);
-    if (bits < (121u << 23)) {                              // below 2^-6: code = floor(value * 512 + 1/2)
-        const uint32_t sig = (bits & 0x7fffffu) | 0x800000u, sh = 141u - (bits >> 23);  // value = sig * 2^(field - 150); sh >= 21
-        code = sh > 31u ? 0u : (sig + (1u << (sh - 1u))) >> sh;  // under 2^-11 (zero and binary32 subnormals too): nothing
+    const uint32_t bits = e4m3_magnitude_bits(y);
+    return e4m3_signed(x, y, bits < kE4m3NormalFrom ? e4m3_code_small(bits) : e4m3_code_normal(bits));
+}
+// Four at once, packed low address first: the rule above, value by value.
+__device__ __forceinline__ uint32_t e4m3_half_up4_any(const float4 v, float scale) {
+    return e4m3_half_up(v.x, scale) | e4m3_half_up(v.y, scale) << 8 | e4m3_half_up(v.z, scale) << 16 | e4m3_half_up(v.w, scale) << 24;
+}
+// The same four codes in about a third of the instructions when the scale is positive and every scaled value is
+// a number of at least 2^-6 in magnitude (a block's amax lands in (224, 448], so smaller ones are rare), which
+// these kernels need: a wave64 vector instruction occupies its SIMD for four cycles, and at 16 bytes in per lane
+// the budget for keeping up with HBM is about 85 of them per kilobyte. What is different: the sign bit is read
+// off fma(x, scale, +0), which is x * scale except that -0 * scale + 0 is +0 (the rule's "x < 0") while a
+// negative product that underflows still rounds to -0; the clamp is an integer minimum on the magnitude bits
+// (an infinity saturates like any large value); and the rebasing constant rides in the rounding add.
+__device__ __forceinline__ uint32_t e4m3_half_up4(const float4 v, float scale) {
+    const float x[4] = {v.x, v.y, v.z, v.w};
+    uint32_t bits[4], mag[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        bits[j] = __float_as_uint(__builtin_fmaf(x[j], scale, 0.0f));
+        mag[j] = bits[j] & 0x7fffffffu;
     }
-    return y != y ? 0u : sign | code;
+    auto lesser = [](uint32_t a, uint32_t b) { return a < b ? a : b; };
+    auto larger = [](uint32_t a, uint32_t b) { return a > b ? a : b; };
+    const uint32_t least = lesser(lesser(mag[0], mag[1]), lesser(mag[2], mag[3])), most = larger(larger(mag[0], mag[1]), larger(mag[2], mag[3]));
+    if (least < kE4m3NormalFrom || most > 0x7f800000u || !(scale > 0.0f)) return e4m3_half_up4_any(v, scale);
+    uint32_t word = 0;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const uint32_t code = (lesser(mag[j], 0x43e00000u /* 448 */) + (0x80000u - ((127u - 7u) << 23))) >> 20;
+        word |= (((bits[j] >> 24) & 0x80u) | code) << (8 * j);
+    }
+    return word;
+}
+
+// Maximum over the eight lanes of a K32 block without leaving the vector unit: neighbours within a quad
+// (lanes ^ 1, ^ 2), then the mirrored half-row, which pairs each quad with the other one of its eight.
+constexpr int kQuadXor1 = 0xB1, kQuadXor2 = 0x4E, kHalfRowMirror = 0x141;  // DPP controls: quad_perm [1,0,3,2], [2,3,0,1], row_half_mirror
+__device__ __forceinline__ float max_over_eight(float v) {
+    int b = __float_as_int(v);
+    v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(b, b, kQuadXor1, 0xf, 0xf, false)));
+    b = __float_as_int(v);
+    v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(b, b, kQuadXor2, 0xf, 0xf, false)));
+    b = __float_as_int(v);
+    return fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(b, b, kHalfRowMirror, 0xf, 0xf, false)));
+}
+__device__ __forceinline__ uint32_t max_bits_over_eight(uint32_t v) {
+    auto larger = [](uint32_t a, uint32_t b) { return a > b ? a : b; };
+    v = larger(v, uint32_t(__builtin_amdgcn_update_dpp(int(v), int(v), kQuadXor1, 0xf, 0xf, false)));
+    v = larger(v, uint32_t(__builtin_amdgcn_update_dpp(int(v), int(v), kQuadXor2, 0xf, 0xf, false)));
+    return larger(v, uint32_t(__builtin_amdgcn_update_dpp(int(v), int(v), kHalfRowMirror, 0xf, 0xf, false)));
 }
 
 // One K32 block per 8 lanes, four values per lane; a workgroup takes 32 consecutive blocks of a row
 // (1024 values), blockIdx.x choosing the piece of the row and blockIdx.y striding over rows, so no
 // thread divides anything. x is contiguous (row r starts at r * 32 * per_row); payload and scales
-// have their own pitches. Two rows are in flight per thread and step.
-__global__ void __launch_bounds__(256) quantize_hidden_kernel(const float* __restrict__ x, long rows, long per_row,
+// have their own pitches; `total` blocks exist (the last row may be short when the host has cut one long
+// array into rows). Four rows are in flight per thread and step.
+//
+// A block of numbers (no NaN, no infinity: its largest magnitude pattern is below 0x7f800000) takes the
+// scale from the bit pattern: with amax = 1.f * 2^(field - 127) the rule's frexp exponent is field - 126 and
+// its mantissa exceeds 0.875 exactly when f exceeds 0.75, so s = field - 8 plus the carry of f + 0.25,
+// floored at 0 (subnormal and zero amax land there); 254 cannot be reached. Any other block goes the long way.
+constexpr int kQuantRowsInFlight = 4;
+__global__ void __launch_bounds__(256) quantize_hidden_kernel(const float* __restrict__ x, long rows, long per_row, long total,
                                                               uint8_t* __restrict__ payload, size_t payload_pitch,
                                                               uint8_t* __restrict__ scales, size_t scales_pitch,
                                                               float* __restrict__ scale_inv) {
     const uint32_t sub = threadIdx.x & 7;
     const long c = long(blockIdx.x) * 32 + (threadIdx.x >> 3);
-    const bool in_row = c < per_row;  // the same for all eight lanes of a block, so the shuffles below see whole blocks
+    const bool in_row = c < per_row;  // the same for all eight lanes of a block, so the exchanges below see whole blocks
     // NaNs take no part in amax. They are zeroed first: a signalling NaN would come out of the
     // hardware maximum as a quiet one and wipe what was gathered before it.
     auto mag = [](float f) { return f != f ? 0.0f : fabsf(f); };
-    auto finish = [&](long r, const float4 v) {
-        float amax = fmaxf(fmaxf(mag(v.x), mag(v.y)), fmaxf(mag(v.z), mag(v.w)));
-#pragma unroll
-        for (int d = 4; d; d >>= 1) amax = fmaxf(amax, __shfl_xor(amax, d));
-        const uint32_t s = q0_scale_byte(amax);
+    auto finish = [&](long r, float4 v, bool live) {
+        if (!live) v = make_float4(0.f, 0.f, 0.f, 0.f);
+        const uint32_t m0 = __float_as_uint(v.x) & 0x7fffffffu, m1 = __float_as_uint(v.y) & 0x7fffffffu,
+                       m2 = __float_as_uint(v.z) & 0x7fffffffu, m3 = __float_as_uint(v.w) & 0x7fffffffu;
+        auto larger = [](uint32_t a, uint32_t b) { return a > b ? a : b; };
+        const uint32_t most = max_bits_over_eight(larger(larger(m0, m1), larger(m2, m3))), field = (most + 0x1fffffu) >> 23;
+        uint32_t s = field > 8u ? field - 8u : 0u;
+        if (most >= 0x7f800000u) {  // the same answer in all eight lanes of the block
+            const float amax = max_over_eight(fmaxf(fmaxf(mag(v.x), mag(v.y)), fmaxf(mag(v.z), mag(v.w))));
+            s = q0_scale_byte(amax);
+        }
         // 2^(127 - s): exponent field 254 - s; s = 254 is 2^-127, the subnormal with the top mantissa bit
         const float scale = __uint_as_float(s == 254u ? 0x00400000u : (254u - s) << 23);
-        if (!in_row) return;
-        if (payload)
-            *reinterpret_cast<uint32_t*>(payload + r * payload_pitch + c * 32 + sub * 4) =
-                e4m3_half_up(v.x, scale) | e4m3_half_up(v.y, scale) << 8 | e4m3_half_up(v.z, scale) << 16 | e4m3_half_up(v.w, scale) << 24;
+        if (!live) return;
+        if (payload) *reinterpret_cast<uint32_t*>(payload + r * payload_pitch + c * 32 + sub * 4) = e4m3_half_up4(v, scale);
         if (sub == 0) {
             if (scales) scales[r * scales_pitch + c] = uint8_t(s);
             if (scale_inv) scale_inv[r * per_row + c] = scale;
         }
     };
-    const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
+    // A set is kQuantRowsInFlight rows, gridDim.y apart. The next set is asked for before this one is worked on:
+    // the arithmetic of a set (some 300 vector instructions, four cycles each) is as long as a memory round
+    // trip, and waves that all load, then all compute, leave HBM idle half of the time.
     const long step = gridDim.y;
-    for (long r = blockIdx.y; r < rows; r += 2 * step) {  // uniform over the workgroup
-        const long r2 = r + step;
-        const float4 v = in_row ? *reinterpret_cast<const float4*>(x + ((r * per_row + c) * 32 + sub * 4)) : zero;
-        const float4 v2 = in_row && r2 < rows ? *reinterpret_cast<const float4*>(x + ((r2 * per_row + c) * 32 + sub * 4)) : zero;
-        finish(r, v);
-        if (r2 < rows) finish(r2, v2);
+    auto fetch = [&](long r, float4 (&v)[kQuantRowsInFlight], bool (&live)[kQuantRowsInFlight]) {
+#pragma unroll
+        for (int j = 0; j < kQuantRowsInFlight; ++j) {
+            const long rj = r + j * step;
+            live[j] = in_row && rj < rows && rj * per_row + c < total;
+            // Every lane loads, a lane without a block the array's first one: a load under a condition would make
+            // the wait ahead of the arithmetic a wait for everything in flight, this set's successor included.
+            v[j] = *reinterpret_cast<const float4*>(x + ((live[j] ? rj * per_row + c : 0) * 32 + sub * 4));
+        }
+    };
+    float4 v[kQuantRowsInFlight], ahead[kQuantRowsInFlight];
+    bool live[kQuantRowsInFlight], live_ahead[kQuantRowsInFlight];
+    fetch(blockIdx.y, v, live);
+    for (long r = blockIdx.y; r < rows; r += kQuantRowsInFlight * step) {  // uniform over the workgroup
+        fetch(r + kQuantRowsInFlight * step, ahead, live_ahead);       // nothing is live past the last row
+#pragma unroll
+        for (int j = 0; j < kQuantRowsInFlight; ++j)
+            if (r + j * step < rows) finish(r + j * step, v[j], live[j]);
+#pragma unroll
+        for (int j = 0; j < kQuantRowsInFlight; ++j) {
+            v[j] = ahead[j];
+            live[j] = live_ahead[j];
+        }
     }
 }
 
@@ -156,8 +238,7 @@ __global__ void __launch_bounds__(256) encode_hidden_kernel(const float* __restr
         if (i + 4 <= n_elem) {
             const float4 v = *reinterpret_cast<const float4*>(x + i);
             const float s = scale_inv[i >> 5];
-            *reinterpret_cast<uint32_t*>(payload + i) = e4m3_half_up(v.x, s) | e4m3_half_up(v.y, s) << 8 |
-                                                        e4m3_half_up(v.z, s) << 16 | e4m3_half_up(v.w, s) << 24;
+            *reinterpret_cast<uint32_t*>(payload + i) = e4m3_half_up4(v, s);
         } else {
             for (int64_t j = i; j < n_elem; ++j) payload[j] = uint8_t(e4m3_half_up(x[j], scale_inv[j >> 5]));
         }

@@ -147,6 +147,44 @@ def test_elementwise_kernels_on_unaligned_pointers_and_short_arrays():
             assert np.array_equal(y.to_host(np.uint16)[shift:shift + n], O.bf16_rne_nan(back[shift:])), (n, shift)
 
 
+def test_wire_quantizer_on_every_exponent_and_code_boundary():
+    """The kernels take the scale and the codes off the bit patterns where a block holds only numbers. Every
+    binary32 exponent with the mantissas around the scale rule's 0.875 threshold as a block's amax, and every
+    E4M3 value, every midpoint between neighbours and the binary32 numbers either side of it under scale 1
+    (a 400.0 leads those blocks), both signs: the same bytes as the CPU rule."""
+    rng = np.random.default_rng(14)
+    fields = np.arange(0, 255, dtype=np.uint32)
+    mants = np.concatenate([np.array([0, 1, 0x3fffff, 0x400000, 0x5fffff, 0x600000, 0x600001, 0x7fffff], np.uint32),
+                            rng.integers(0, 1 << 23, 24).astype(np.uint32)])
+    amax = ((fields[:, None] << 23) | mants[None, :]).reshape(-1).astype(np.uint32).view(np.float32)
+    a = (rng.standard_normal((amax.size, 32)).astype(np.float32) * amax[:, None]).astype(np.float32)
+    a[np.abs(a) > amax[:, None]] = 0
+    a[:, 5] = amax
+    a[::2, 5] *= -1
+    codes = np.arange(0, 0x7f, dtype=np.uint32)
+    value = np.where(codes < 8, codes * 2.0 ** -9, (1 + (codes & 7) / 8) * 2.0 ** ((codes >> 3).astype(np.int64) - 7)).astype(np.float32)
+    mid = ((value[:-1].astype(np.float64) + value[1:]) / 2).astype(np.float32)
+    cand = np.concatenate([value, mid, np.nextafter(mid, np.float32(0)), np.nextafter(mid, np.float32(1e9)),
+                           rng.uniform(0, 448, 4000).astype(np.float32), np.exp2(rng.uniform(-12, 8.8, 4000)).astype(np.float32)])
+    cand = np.resize(cand, (cand.size + 30) // 31 * 31).reshape(-1, 31) * np.where(rng.random(((cand.size + 30) // 31, 31)) < 0.5, -1, 1)
+    b = np.concatenate([np.full((cand.shape[0], 1), 400.0, np.float32), cand.astype(np.float32)], axis=1)
+    x = np.concatenate([a.reshape(-1), b.reshape(-1)])
+    x = np.resize(x, (x.size + 4095) // 4096 * 4096).reshape(-1, 4096).astype(np.float32)
+    with np.errstate(all="ignore"):
+        ref_p, ref_s = O.q0_quantize(x)
+        _, ref_inv = O.q0_scales(x)
+    rows = x.shape[0]
+    dx, frame, ds, dinv, dp = dev(x), D(rows * 4224 + 64), D(rows * 128), D(rows * 512), D(rows * 4096)
+    glue.quantize_hidden(dx.ptr, rows, 4096, frame.ptr, 4224, frame.ptr + 4096, 4224)
+    got = frame.to_host(np.uint8)[: rows * 4224].reshape(rows, 4224)
+    assert np.array_equal(got[:, 4096:], ref_s) and np.array_equal(got[:, :4096], ref_p)
+    glue.quant_scales(dx.ptr, rows * 128, ds.ptr, dinv.ptr)
+    glue.quantize_hidden_fp8(dx.ptr, dinv.ptr, dp.ptr, rows * 4096)
+    assert np.array_equal(ds.to_host(np.uint8).reshape(rows, 128), ref_s)
+    assert np.array_equal(dinv.to_host(np.uint32), ref_inv.view(np.uint32))
+    assert np.array_equal(dp.to_host(np.uint8).reshape(rows, 4096), ref_p)
+
+
 def test_wire_quantizer_row_shapes():
     """Rows shorter than a workgroup's 1024 values, rows that are not a multiple of it, and pitched outputs: the
     same bytes as the CPU rule row by row."""
