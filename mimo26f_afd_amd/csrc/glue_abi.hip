@@ -50,8 +50,14 @@ int m26c_router_topk(const float* logits, const float* bias, int rows, int n_exp
     if (n_experts <= 0 || n_experts > 64 * kRouterPerLane || n_experts % 32 || top_k <= 0 || top_k > n_experts ||
         top_k > 64 || !logits || !bias || !idx_out || !w_out)
         return 1;
-    router_topk_kernel<<<(rows + 3) / 4, kThreads, 0, hipStream_t(stream)>>>(logits, bias, rows, n_experts, top_k, idx_out,
-                                                                            w_out);
+    const dim3 grid((rows + 3) / 4);
+    hipStream_t st = hipStream_t(stream);
+    const int per = (n_experts + 63) / 64;  // a lane's share, rounded up to a compiled size
+    if (per <= 1) router_topk_kernel<1><<<grid, kThreads, 0, st>>>(logits, bias, rows, n_experts, top_k, idx_out, w_out);
+    else if (per <= 2) router_topk_kernel<2><<<grid, kThreads, 0, st>>>(logits, bias, rows, n_experts, top_k, idx_out, w_out);
+    else if (per <= 4) router_topk_kernel<4><<<grid, kThreads, 0, st>>>(logits, bias, rows, n_experts, top_k, idx_out, w_out);
+    else if (per <= 8) router_topk_kernel<8><<<grid, kThreads, 0, st>>>(logits, bias, rows, n_experts, top_k, idx_out, w_out);
+    else router_topk_kernel<kRouterPerLane><<<grid, kThreads, 0, st>>>(logits, bias, rows, n_experts, top_k, idx_out, w_out);
     return launched();
 }
 

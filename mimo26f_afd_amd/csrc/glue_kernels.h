@@ -13,30 +13,50 @@
 namespace m26g {
 
 // ---- routing ------------------------------------------------------------------------------------
-// One wave per row; lane l holds experts l, l+64, ... (at most 16 of them, n_experts <= 1024).
+// One wave per row; lane l holds experts l, l+64, ... (PER of them, n_experts <= 64 * PER <= 1024).
 // Scores and the selection run in binary64 like the reference; the k selections are k wave-wide
 // arg-max rounds on (score + bias, lower id wins ties). Weights: unbiased score / sum, the sum taken
 // in selection order, rounded to binary32.
+//
+// The rounds are a chain of dependent steps, so the wave-wide arg-max stays inside the vector unit: DPP moves
+// within a row of sixteen lanes (neighbours in a quad, the mirrored half-row, the mirrored row), then the last
+// lane of a row handed to the next row and the last lane of the second row to the upper two, after which lane
+// 63 holds the winner and a lane read makes it uniform. Through the LDS crossbar (the shuffle intrinsics) the
+// same eight rounds took three times as long.
 constexpr int kRouterPerLane = 16;
 
-__device__ __forceinline__ void wave_argmax(double& v, int& i) {
-#pragma unroll
-    for (int d = 32; d; d >>= 1) {
-        const double ov = __shfl_xor(v, d);
-        const int oi = __shfl_xor(i, d);
-        if (ov > v || (ov == v && oi < i)) { v = ov; i = oi; }
-    }
+struct Best {
+    double v;
+    int i;
+};
+__device__ __forceinline__ Best better(Best a, Best b) { return (b.v > a.v || (b.v == a.v && b.i < a.i)) ? b : a; }
+template <int CTRL, int ROWS>
+__device__ __forceinline__ Best best_from(Best a) {  // lanes of rows outside ROWS get their own value back
+    const int lo = __double2loint(a.v), hi = __double2hiint(a.v);
+    return Best{__hiloint2double(__builtin_amdgcn_update_dpp(hi, hi, CTRL, ROWS, 0xf, false), __builtin_amdgcn_update_dpp(lo, lo, CTRL, ROWS, 0xf, false)),
+                __builtin_amdgcn_update_dpp(a.i, a.i, CTRL, ROWS, 0xf, false)};
+}
+__device__ __forceinline__ Best wave_best(Best a) {
+    a = better(a, best_from<0xB1, 0xf>(a));   // quad_perm [1,0,3,2]
+    a = better(a, best_from<0x4E, 0xf>(a));   // quad_perm [2,3,0,1]
+    a = better(a, best_from<0x141, 0xf>(a));  // row_half_mirror
+    a = better(a, best_from<0x140, 0xf>(a));  // row_mirror: every lane of a row holds the row's best
+    a = better(a, best_from<0x142, 0xa>(a));  // row_bcast15 into rows 1 and 3
+    a = better(a, best_from<0x143, 0xc>(a));  // row_bcast31 into rows 2 and 3: lane 63 holds the wave's best
+    return Best{__hiloint2double(__builtin_amdgcn_readlane(__double2hiint(a.v), 63), __builtin_amdgcn_readlane(__double2loint(a.v), 63)),
+                __builtin_amdgcn_readlane(a.i, 63)};
 }
 
+template <int PER>
 __global__ void __launch_bounds__(256) router_topk_kernel(const float* __restrict__ logits, const float* __restrict__ bias,
                                                           int rows, int n_experts, int top_k, int* __restrict__ idx_out,
                                                           float* __restrict__ w_out) {
     const int lane = threadIdx.x & 63, row = blockIdx.x * 4 + (threadIdx.x >> 6);
     if (row >= rows) return;
     const float* lrow = logits + size_t(row) * n_experts;
-    double score[kRouterPerLane], sel[kRouterPerLane];
+    double score[PER], sel[PER];
 #pragma unroll
-    for (int j = 0; j < kRouterPerLane; ++j) {
+    for (int j = 0; j < PER; ++j) {
         const int e = lane + 64 * j;
         if (e < n_experts) {
             score[j] = 1.0 / (1.0 + exp(-double(lrow[e])));
@@ -49,22 +69,22 @@ __global__ void __launch_bounds__(256) router_topk_kernel(const float* __restric
     double wsum = 0.0, mine = 0.0;  // lane k keeps the k-th chosen score
     int mine_id = 0;
     for (int k = 0; k < top_k; ++k) {
-        double v = -INFINITY;
-        int i = 0x7fffffff;
+        Best b{-INFINITY, 0x7fffffff};
 #pragma unroll
-        for (int j = 0; j < kRouterPerLane; ++j) {  // ascending ids: a strict > keeps the lower id on ties
-            const int e = lane + 64 * j;
-            if (e < n_experts && sel[j] > v) { v = sel[j]; i = e; }
-        }
-        wave_argmax(v, i);
-        const int owner = i & 63, slot = i >> 6;
+        for (int j = 0; j < PER; ++j)  // ascending ids: a strict > keeps the lower id on ties; absent experts hold -inf
+            if (sel[j] > b.v) b = Best{sel[j], lane + 64 * j};
+        b = wave_best(b);              // the same in every lane, and known to be
+        const int owner = b.i & 63, slot = b.i >> 6;
         double s = 0.0;
 #pragma unroll
-        for (int j = 0; j < kRouterPerLane; ++j)
-            if (j == slot && lane == owner) { s = score[j]; sel[j] = -INFINITY; }
-        s = __shfl(s, owner);
+        for (int j = 0; j < PER; ++j)
+            if (j == slot) {
+                s = __hiloint2double(__builtin_amdgcn_readlane(__double2hiint(score[j]), owner),
+                                     __builtin_amdgcn_readlane(__double2loint(score[j]), owner));
+                if (lane == owner) sel[j] = -INFINITY;
+            }
         wsum += s;
-        if (lane == k) { mine = s; mine_id = i; }
+        if (lane == k) { mine = s; mine_id = b.i; }
     }
     if (lane < top_k) {
         idx_out[size_t(row) * top_k + lane] = mine_id;
