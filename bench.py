@@ -292,6 +292,72 @@ def run_rank_share(torch, dev, b1, synth, O):
     return out
 
 
+def run_coordinator_kernels(torch, dev):
+    """The kernels either side of the path (routing, wire quantizer, frame fill, rank sum, residual add, BF16 cast)
+    at the prefill chunk's and the decode batch's row counts: ten launches between two events on torch's stream,
+    median of 15 such pairs, the algorithmic bytes of one launch over that time. Each is a pass over a few bytes
+    per value, so HBM is the bound; up to about 250 MB a working set also lives in the last-level cache between
+    the repeats, and a launch costs about 4 us whatever it moves."""
+    from mimo26f_afd_amd import glue
+    st = torch.cuda.current_stream().cuda_stream
+    H, E, K, PITCH, REPEAT, PAIRS = 4096, 256, 8, 4224, 10, 15
+
+    def timed(fn):
+        for _ in range(3):
+            fn()
+        torch.cuda.synchronize()
+        ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(PAIRS)]
+        for a, b in ev:
+            a.record()
+            for _ in range(REPEAT):
+                fn()
+            b.record()
+        torch.cuda.synchronize()
+        return float(np.median([a.elapsed_time(b) for a, b in ev])) / REPEAT
+
+    out = {"peak_GBps": HBM_PEAK_GBS, "protocol": f"{REPEAT} launches per event pair, median of {PAIRS} pairs; bytes = what one launch must read and write",
+           "rows": {}}
+    for T in (8192, 128):
+        g = torch.Generator(device="cpu").manual_seed(0x26AFD + T)
+        x = torch.randn(T, H, generator=g).to(dev)
+        a = torch.randn(T, H, generator=g).to(dev)
+        logits = torch.randn(T, E, generator=g).to(dev)
+        bias = torch.zeros(E, device=dev)
+        idx = torch.empty(T, K, dtype=torch.int32, device=dev)
+        w = torch.empty(T, K, device=dev)
+        frame = torch.empty(T * PITCH + 4096, dtype=torch.uint8, device=dev)
+        payload = torch.empty(T, H, dtype=torch.uint8, device=dev)
+        scales = torch.empty(T, H // 32, dtype=torch.uint8, device=dev)
+        sinv = torch.empty(T * H // 32, device=dev)
+        routes = torch.empty(T * K * 12, dtype=torch.uint8, device=dev)
+        part = [torch.randn(T, H, generator=g).to(dev).to(torch.bfloat16) for _ in range(4)]
+        acc = torch.empty(T, H, device=dev)
+        y16 = torch.empty(T, H, dtype=torch.int16, device=dev)
+        n = T * H
+        glue.router_topk(logits.data_ptr(), bias.data_ptr(), T, E, K, idx.data_ptr(), w.data_ptr(), st)
+        glue.quant_scales(x.data_ptr(), n // 32, scales.data_ptr(), sinv.data_ptr(), st)
+        cases = {
+            "m26c_router_topk": (lambda: glue.router_topk(logits.data_ptr(), bias.data_ptr(), T, E, K, idx.data_ptr(), w.data_ptr(), st),
+                                 T * E * 4 + T * K * 8),
+            "m26c_quantize_hidden (into frame rows)": (lambda: glue.quantize_hidden(x.data_ptr(), T, H, frame.data_ptr(), PITCH, frame.data_ptr() + H, PITCH, st),
+                                                       n * 4 + T * (H + H // 32)),
+            "m26c_quant_scales": (lambda: glue.quant_scales(x.data_ptr(), n // 32, scales.data_ptr(), sinv.data_ptr(), st), n * 4 + n // 32 * 5),
+            "m26_quantize_hidden_fp8": (lambda: glue.quantize_hidden_fp8(x.data_ptr(), sinv.data_ptr(), payload.data_ptr(), n, st), n * 4 + n // 32 * 4 + n),
+            "m26c_frame_fill": (lambda: glue.frame_fill(idx.data_ptr(), w.data_ptr(), payload.data_ptr(), scales.data_ptr(), T, K, H, routes.data_ptr(),
+                                                        frame.data_ptr(), PITCH, st), 2 * T * (H + H // 32) + T * K * (8 + 12)),
+            "m26c_rank_sum_bf16": (lambda: glue.rank_sum_bf16(*[q.data_ptr() for q in part], acc.data_ptr(), n, st), n * 8 + n * 4),
+            "m26c_add_inplace": (lambda: glue.add_inplace(acc.data_ptr(), a.data_ptr(), n, st), n * 12),
+            "m26c_f32_to_bf16": (lambda: glue.f32_to_bf16(x.data_ptr(), y16.data_ptr(), n, st), n * 6),
+        }
+        rows = {}
+        for name, (fn, nbytes) in cases.items():
+            ms = timed(fn)
+            gbs = nbytes / (ms * 1e-3) / 1e9
+            rows[name] = {"us": ms * 1e3, "bytes": nbytes, "GBps": gbs, "frac_of_hbm_peak": gbs / HBM_PEAK_GBS}
+        out["rows"][str(T)] = rows
+    return out
+
+
 def stack_reference_rows(seed, layer, payload, scales, ids, weights, O, synth):
     """The CPU rule's BF16 rows for a few tokens of one stack layer, its touched experts regenerated on the host."""
     pools = []
@@ -402,6 +468,8 @@ def main():
                     help="profiling aid: run only the prefill measurement and print its object")
     ap.add_argument("--no-stack", action="store_true", help="skip the 48-layer resident stack (configs[4]) object")
     ap.add_argument("--no-rank-share", action="store_true", help="skip the rank-share object (configs[0], configs[1], the reference's gate sweep)")
+    ap.add_argument("--no-coordinator-kernels", action="store_true", help="skip the object that times the kernels either side of the path")
+    ap.add_argument("--only-coordinator-kernels", action="store_true", help="profiling aid: run only that leg and print its object")
     ap.add_argument("--only-rank-share", action="store_true", help="profiling aid: run only the rank-share leg and print its object")
     ap.add_argument("--no-variants", action="store_true",
                     help="profiling aid: skip the opt-in forms (fused combine, BF16 per-route rows) sampled beside the default, so a kernel "
@@ -432,6 +500,9 @@ def main():
         torch.cuda.synchronize()
         del src, dst
         torch.cuda.empty_cache()
+    if args.only_coordinator_kernels:
+        print(json.dumps(run_coordinator_kernels(torch, dev)), flush=True)
+        return
     if args.only_rank_share:
         print(json.dumps(run_rank_share(torch, dev, b1, synth, O)), flush=True)
         return
@@ -528,6 +599,11 @@ def main():
             "mfma_only_TFLOPs_after_40_launches": held["tflops_last"]}
         if fc1_ghz:
             line["prefill"]["roofline"]["frac_at_clock"] = fc1_tf / (MFMA_FP8_PEAK_TFLOPS * fc1_ghz / NOMINAL_GHZ)
+    if not args.no_coordinator_kernels:
+        try:
+            line["coordinator_kernels"] = run_coordinator_kernels(torch, dev)
+        except Exception as e:  # a leg beside the headline: reported, never fatal
+            line["coordinator_kernels"] = {"error": f"{type(e).__name__}: {e}"}
     if not args.no_rank_share:
         try:
             t0 = time.time()

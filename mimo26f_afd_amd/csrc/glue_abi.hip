@@ -30,11 +30,12 @@ int launch_quantize(const float* x, long rows, long per_row, uint8_t* payload, s
         payload_pitch = 1024;
         scales_pitch = 32;
     }
-    // About four workgroups per compute unit, each walking several sets of rows with the next set's loads in flight.
-    const long pieces = (per_row + 31) / 32, lines = (rows + kQuantRowsInFlight - 1) / kQuantRowsInFlight;
+    // About four workgroups per compute unit, each walking several sets of rows with the next set's loads in flight;
+    // with fewer rows than that, a workgroup per row (a thread's other three rows fall past the end).
+    const long pieces = (per_row + 31) / 32;
     if (pieces > 0x7fffffffL) return 1;
     long walkers = pieces >= 1024 ? 1 : 1024 / pieces;
-    walkers = walkers < lines ? walkers : lines;
+    walkers = walkers < rows ? walkers : rows;
     quantize_hidden_kernel<<<dim3(unsigned(pieces), unsigned(walkers)), kThreads, 0, hipStream_t(stream)>>>(
         x, rows, per_row, total, payload, payload_pitch, scales, scales_pitch, scale_inv);
     return launched();
