@@ -10,10 +10,16 @@ extern "C" {
 #endif
 
 /* CRC32C (Castagnoli, reflected polynomial 0x82F63B78) update over host bytes, the L4 frame checksum
- * of crates/mimo26-wire/src/crc32c.rs:107-140: pass state = 0xFFFFFFFF first, chain the returned
+ * of crates/mimo26-wire/src/crc32c.rs:107-140 (the host's CRC32C instruction where it has one, as there:
+ * crc32c.rs:48-66, 86-104): pass state = 0xFFFFFFFF first, chain the returned
  * state over further segments, and invert the last one. m26w_crc32c_update(~0, "123456789", 9)
  * inverted is 0xE3069283. */
 uint32_t m26w_crc32c_update(uint32_t state, const uint8_t* data, size_t n);
+
+/* The same function by table look-ups only: what m26w_crc32c_update falls back to on a host without a
+ * CRC32C instruction, exported so that the instruction path can be compared with it (the reference keeps
+ * its byte-wise table walk beside update_sse42 for the same purpose, crc32c.rs:37-46, 203-216). */
+uint32_t m26w_crc32c_update_portable(uint32_t state, const uint8_t* data, size_t n);
 
 /* The route gathering of serve_b1_view (serve.rs:219-232) on the device, for a request frame whose
  * body lies in device memory: `descriptors_dev` = rows x 40-byte row descriptors, `routes_dev` =

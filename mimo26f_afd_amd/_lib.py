@@ -12,6 +12,7 @@ _vp, _sz, _cp = C.c_void_p, C.c_size_t, C.c_char_p
 # name -> (restype, argtypes); every symbol include/m26s_b1.h, include/m26c_glue.h and include/m26w_frame.h declare
 SIGNATURES = {
     "m26w_crc32c_update": (C.c_uint32, [C.c_uint32, _vp, _sz]),
+    "m26w_crc32c_update_portable": (C.c_uint32, [C.c_uint32, _vp, _sz]),
     "m26w_request_routes_dev": (C.c_int, [_vp, _vp, C.c_uint32, C.c_uint32, _vp, _vp, _vp, _vp]),
     "m26w_stage_rows_dev": (C.c_int, [_vp, _vp, _sz, _vp]),
     "m26c_router_topk": (C.c_int, [_vp, _vp, C.c_int, C.c_int, C.c_int, _vp, _vp, _vp]),

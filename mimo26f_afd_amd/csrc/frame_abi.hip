@@ -47,7 +47,10 @@ __global__ void arm_fault_kernel(uint32_t* fault) { *fault = 0xffffffffu; }
 __global__ void settle_fault_kernel(uint32_t* fault) { if (*fault == 0xffffffffu) *fault = 0; }
 }  // namespace
 
-extern "C" uint32_t m26w_crc32c_update(uint32_t state, const uint8_t* data, size_t n) {
+// The table walk: eight bytes per step through eight 256-entry tables. The fallback where the host has no
+// CRC32C instruction, and the checker the instruction path is compared with (crates/mimo26-wire/src/
+// crc32c.rs:37-46 keeps its byte-wise walk for the same two purposes).
+extern "C" uint32_t m26w_crc32c_update_portable(uint32_t state, const uint8_t* data, size_t n) {
     static const CrcTables tables;
     const uint32_t (*t)[256] = tables.t;
     uint32_t c = state;
@@ -63,6 +66,82 @@ extern "C" uint32_t m26w_crc32c_update(uint32_t state, const uint8_t* data, size
     }
     while (n--) c = (c >> 8) ^ t[0][(c ^ *data++) & 0xffu];
     return c;
+}
+
+namespace {
+// The x86-64 CRC32C instruction (SSE4.2; the reference's update_sse42, crc32c.rs:48-66) retires eight bytes
+// every three cycles on one dependency chain and one a cycle over three independent ones, so long inputs
+// are walked as three stripes side by side and the three states are joined afterwards: appending m bytes to
+// a message multiplies its state by x^(8m) modulo the polynomial, a linear map over GF(2) that four
+// 256-entry tables apply to a 32-bit state.
+constexpr size_t kStripe = 4096;  // bytes per stripe; a frame's hidden rows alone are 4224 bytes each
+
+struct ShiftTables {
+    uint32_t z[4][256];  // state -> state after kStripe further zero bytes (on raw states, no inversion)
+    static uint32_t times(const uint32_t (&mat)[32], uint32_t vec) {
+        uint32_t sum = 0;
+        for (int i = 0; vec; vec >>= 1, ++i)
+            if (vec & 1u) sum ^= mat[i];
+        return sum;
+    }
+    ShiftTables() {
+        uint32_t op[32], sq[32];
+        op[0] = 0x82F63B78u;  // one zero bit: bit 0 leaves and brings the polynomial in, the others move down
+        for (int i = 1; i < 32; ++i) op[i] = 1u << (i - 1);
+        size_t bits = 1;
+        while (bits < kStripe * 8) {  // kStripe * 8 is a power of two: square up to it
+            for (int i = 0; i < 32; ++i) sq[i] = times(op, op[i]);
+            memcpy(op, sq, sizeof op);
+            bits *= 2;
+        }
+        for (uint32_t b = 0; b < 256; ++b)
+            for (int k = 0; k < 4; ++k) z[k][b] = times(op, b << (8 * k));
+    }
+    uint32_t shift(uint32_t c) const { return z[0][c & 0xff] ^ z[1][(c >> 8) & 0xff] ^ z[2][(c >> 16) & 0xff] ^ z[3][c >> 24]; }
+};
+static_assert((kStripe & (kStripe - 1)) == 0 && kStripe % 8 == 0, "a stripe is a power of two of whole words");
+
+#if defined(__x86_64__)
+__attribute__((target("sse4.2"))) uint32_t crc32c_hw(uint32_t state, const uint8_t* data, size_t n) {
+    static const ShiftTables tables;
+    uint64_t c = state;
+    while (n && (reinterpret_cast<uintptr_t>(data) & 7u)) { c = __builtin_ia32_crc32qi(uint32_t(c), *data++); --n; }
+    while (n >= 3 * kStripe) {
+        uint64_t c1 = 0, c2 = 0;  // a stripe that starts from state 0 contributes its state unchanged: the map is linear
+        const uint8_t* p = data;
+        for (size_t i = 0; i < kStripe; i += 8, p += 8) {
+            uint64_t w0, w1, w2;
+            memcpy(&w0, p, 8);
+            memcpy(&w1, p + kStripe, 8);
+            memcpy(&w2, p + 2 * kStripe, 8);
+            c = __builtin_ia32_crc32di(c, w0);
+            c1 = __builtin_ia32_crc32di(c1, w1);
+            c2 = __builtin_ia32_crc32di(c2, w2);
+        }
+        c = tables.shift(uint32_t(c)) ^ uint32_t(c1);
+        c = tables.shift(uint32_t(c)) ^ uint32_t(c2);
+        data += 3 * kStripe;
+        n -= 3 * kStripe;
+    }
+    while (n >= 8) {
+        uint64_t w;
+        memcpy(&w, data, 8);
+        c = __builtin_ia32_crc32di(c, w);
+        data += 8;
+        n -= 8;
+    }
+    while (n--) c = __builtin_ia32_crc32qi(uint32_t(c), *data++);
+    return uint32_t(c);
+}
+#endif
+}  // namespace
+
+extern "C" uint32_t m26w_crc32c_update(uint32_t state, const uint8_t* data, size_t n) {
+#if defined(__x86_64__)
+    static const bool hw = __builtin_cpu_supports("sse4.2");
+    if (hw) return crc32c_hw(state, data, n);
+#endif
+    return m26w_crc32c_update_portable(state, data, n);
 }
 
 extern "C" int m26w_request_routes_dev(const uint8_t* descriptors_dev, const uint8_t* routes_dev, uint32_t rows,

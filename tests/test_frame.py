@@ -44,6 +44,37 @@ def test_wire_constants_and_pinned_entry_bytes():
         assert F.crc32c(data[lo:hi].copy()) == c ^ 0xFFFFFFFF and F.crc32c(data[lo:hi]) == c ^ 0xFFFFFFFF
 
 
+def test_crc32c_instruction_path_equals_the_table_walk():
+    """m26w_crc32c_update uses the host's CRC32C instruction where there is one, three stripes of 4096 bytes side
+    by side joined by the x^(8 * 4096) map; m26w_crc32c_update_portable is the table walk. Same state for every
+    length around the stripe and triple-stripe boundaries, at every alignment, chained across an arbitrary cut,
+    from an arbitrary starting state, and on a buffer the size of a 4096-row request frame (the reference compares
+    its two paths at 1 MiB and 17.86 MB, crates/mimo26-wire/src/crc32c.rs:203-216). Both paths also get the
+    bit-by-bit value on a 13 KB run, so the joining of stripes is pinned independently of the tables."""
+    from mimo26f_afd_amd._lib import load
+    lib = load()
+    rng = np.random.default_rng(1)
+    buf = rng.integers(0, 256, 128 + 4096 * 4360 + 64, dtype=np.uint8)
+    lengths = [0, 1, 7, 8, 9, 4095, 4096, 4097, 12287, 12288, 12289, 12296, 24576 + 5, 3 * 4096 * 5 + 13, 1 << 20, buf.size - 16]
+    for n in lengths:
+        for off in (0, 1, 3, 8):
+            a = buf[off:off + n]
+            for start in (0xFFFFFFFF, 0, 0x12345678):
+                want = lib.m26w_crc32c_update_portable(start, a.ctypes.data, a.size)
+                assert lib.m26w_crc32c_update(start, a.ctypes.data, a.size) == want, (n, off, start)
+                cut = n // 3
+                head = lib.m26w_crc32c_update(start, a.ctypes.data, cut)
+                assert lib.m26w_crc32c_update(head, a.ctypes.data + cut, n - cut) == want, (n, off, start)
+    run = buf[5:5 + 13000]
+    c = 0xFFFFFFFF
+    for b in run:
+        c ^= int(b)
+        for _ in range(8):
+            c = (c >> 1) ^ (0x82F63B78 if c & 1 else 0)
+    assert lib.m26w_crc32c_update(0xFFFFFFFF, run.ctypes.data, run.size) == c
+    assert lib.m26w_crc32c_update_portable(0xFFFFFFFF, run.ctypes.data, run.size) == c
+
+
 def test_request_round_trip_and_body_accounting():
     for rows in (1, 3, 16):
         frame, payload, scales, ids, w = small_request(rows, request_id=42, layer_id=5, executor_id=2, seq=9)
